@@ -11,6 +11,7 @@ NAMES = {
     "paged_attn": "libmistralrspagedattention.so",
     "core": "libmistralrscuda.so",
     "ext": "libmrs_hip_ext.so",
+    "hybrid": "libmrs_hybrid.so",
 }
 _cache: dict[str, C.CDLL] = {}
 
@@ -38,6 +39,18 @@ def load(key: str) -> C.CDLL:
                 "There is deliberately no fallback path.")
         _cache[key] = C.CDLL(p, mode=C.RTLD_GLOBAL)
     return _cache[key]
+
+
+def host_key() -> str:
+    """The library that serves the host-side cache bookkeeping (`mrs_kv_*`, `mrs_state_pool_*`): libmrs_hip_ext.so and libmrs_hybrid.so both link those objects; a
+    checkout that has only built the small one uses it."""
+    if "ext" in _cache or os.path.exists(path("ext")):
+        try:
+            getattr(load("ext"), "mrs_state_pool_create")
+            return "ext"
+        except (AttributeError, OSError):
+            pass
+    return "hybrid"
 
 
 def sym(key: str, name: str, argtypes, restype=None):

@@ -27,6 +27,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 CXXFLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Wno-unused-value", "-ffp-contract=off",
             "-I" + CSRC, "-I" + os.path.join(os.path.dirname(HERE), "include")]
 
+HYBRID_LIB = "libmrs_hybrid.so"
+PACKED_FP32_OFF = ("-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")  # device code without packed f32 instructions
+
 MMVQ_TYPES = {"q4_0": 2, "q4_1": 3, "q5_0": 6, "q5_1": 7, "q8_0": 8,
               "q2_k": 10, "q3_k": 11, "q4_k": 12, "q5_k": 13, "q6_k": 14}
 
@@ -57,7 +60,7 @@ def libraries():
         "libmistralrsquant.so": ["quant_ops.hip", "mmq.hip", "moe.hip", "gemv.hip", "hqq.hip"],
         "libmistralrscuda.so": ["core_ops.hip", "sampling.hip"],
         "libmrs_hip_ext.so": ["ext_decode.hip", "ext_dec.hip", "ext_dec_mm.hip", "ext_gemm.hip", "ext_gemm_qi.hip", "ext_attn_prefill.hip", "ext_comm.hip", "ext_p2p.hip", "ext_hqq_gemv.hip", "ext_isq.hip", "ext_prefetch.hip", "ext_gemm_lt.hip",
-                              "host/runtime.cpp", "host/kv_cache_manager.cpp"],
+                              "host/runtime.cpp", "host/kv_cache_manager.cpp", "host/state_pool.cpp"],
     }
     # experiment knob (default off): MRS_DECODE_MIN_WAVES=4 caps the decode GEMV kernels at 128 VGPRs (csrc/ext_decode.hip); use with --force
     decode_defs = {"ext_decode.hip": (f"-DMRS_DECODE_MIN_WAVES={os.environ['MRS_DECODE_MIN_WAVES']}",)} if os.environ.get("MRS_DECODE_MIN_WAVES") else {}
@@ -67,6 +70,10 @@ def libraries():
         for s in srcs:
             if os.path.exists(os.path.join(CSRC, s)):
                 libs.setdefault(lib, []).append(_tu(s, os.path.basename(os.path.splitext(s)[0]) + ".o", decode_defs.get(s, ())))
+    # layer-list ("hybrid") decoders in their checkpoint dtype: a library of its own, so that serving such a model compiles four files, not the quantized stack.
+    # It carries the host-side cache bookkeeping too (the same objects libmrs_hip_ext.so links).
+    libs[HYBRID_LIB] = [_tu(s, os.path.basename(os.path.splitext(s)[0]) + ".o", PACKED_FP32_OFF if s.endswith(".hip") else ())
+                        for s in ("hyb_gemm.hip", "hyb_kernels.hip", "host/kv_cache_manager.cpp", "host/state_pool.cpp")]
     return libs
 
 
@@ -110,15 +117,23 @@ def _compile(src, obj, defines, force, hdr_m):
     return o, True
 
 
-def build(jobs: int | None = None, force: bool = False, verbose: bool = True) -> dict:
+def build(jobs: int | None = None, force: bool = False, verbose: bool = True, only=None) -> dict:
+    """`only`: names of the libraries to build (default: all)."""
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIB, exist_ok=True)
     libs = libraries()
+    if only:
+        libs = {k: v for k, v in libs.items() if k in only}
     hdr_m = _headers_mtime()
     jobs = jobs or min(16, os.cpu_count() or 4)
     out = {}
     with cf.ThreadPoolExecutor(jobs) as ex:
-        futs = {name: [ex.submit(_compile, *tu, force, hdr_m) for tu in tus] for name, tus in libs.items()}
+        once = {}  # a translation unit that two libraries link is compiled once
+        for tus in libs.values():
+            for tu in tus:
+                if tu not in once:
+                    once[tu] = ex.submit(_compile, *tu, force, hdr_m)
+        futs = {name: [once[tu] for tu in tus] for name, tus in libs.items()}
         for name, fl in sorted(futs.items(), key=lambda kv: kv[0] == "libmrs_hip_ext.so"):  # ext links last
             res = [f.result() for f in fl]
             objs = [o for o, _ in res]
@@ -143,6 +158,7 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("-j", type=int, default=None)
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--only", default=None, help="comma-separated library names (default: all)")
     a = ap.parse_args()
-    for k, v in build(a.j, a.force).items():
+    for k, v in build(a.j, a.force, only=a.only.split(",") if a.only else None).items():
         print(k, "->", v)

@@ -1,0 +1,299 @@
+// hyb_gemm.hip -- plain dense products for models whose weights stay in their checkpoint dtype (bf16, or f32 for the all-f32 serving mode):
+//   C[M, N] (f32)  (+)=  A[M, K] . W[N, K]^T          A, W in T = bf16 | f32, both K-contiguous ("x W^T": weights stored [out, in])
+// Two kernels per dtype:
+//   * gemm_tile_kernel: 64 x 64 output tile per workgroup of four waves, K in steps of 32 through LDS; bf16 operands go to v_mfma_f32_32x32x16_bf16 (one 32 x 32
+//     quadrant per wave), f32 operands to a 4 x 4 register block per thread on the vector ALU (true f32: products and sums in f32, k ascending).  Grouped form: the rows
+//     are sorted by group, group g owns rows [bounds[g], bounds[g + 1]) and the weight slab W + g * wstride (mixture-of-experts layers: one launch for all experts,
+//     the bounds are read on the device, tiles past a group's rows leave).
+//   * gemv_rows_kernel: M <= 8 rows (decode steps): one wave per output column streams the weight row with 16-byte loads, f32 accumulation per activation row,
+//     butterfly sum.  Grouped form: every activation row has its own weight slab (row_group[m]).
+// f32 results only: the consumers (residual sum, norms, recurrences, routers) are f32 anyway; what a consumer feeds into the next product it rounds itself, once.
+#include "common.cuh"
+
+namespace mrs {
+namespace hyb {
+
+typedef short bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct GemmArgs {
+  const void *A;
+  const void *W;
+  float *C;
+  int M, N, K, lda, ldw, ldc;
+  int accumulate;            // C += instead of C =
+  const int *bounds;         // grouped: [groups + 1] row bounds (device), else null
+  long long wstride;         // elements between the groups' weight slabs
+  int vec_ok;                // K, lda, ldw multiples of 8 (bf16) / 4 (f32) and 16-byte aligned bases: vector loads
+};
+
+constexpr int BM = 64, BN = 64, BK = 32;
+
+template <class T> struct TileLoad;
+template <> struct TileLoad<bf16_t> {
+  // 64 rows x 32 k of bf16 = 256 threads x 8 values
+  static __device__ __forceinline__ void load(const bf16_t *base, int ld, int row0, int rows_end, int k0, int K, int vec_ok, int tid, uint16_t (*dst)[BK + 8]) {
+    const int r = tid >> 2, kc = (tid & 3) * 8;
+    const int row = row0 + r;
+    int4 v = make_int4(0, 0, 0, 0);
+    if (row < rows_end) {
+      const bf16_t *p = base + (size_t)row * ld + k0 + kc;
+      if (vec_ok && k0 + kc + 8 <= K) v = *(const int4 *)p;
+      else {
+        uint16_t t[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = (k0 + kc + j < K) ? p[j].v : (uint16_t)0;
+        v = make_int4((int)(t[0] | ((unsigned)t[1] << 16)), (int)(t[2] | ((unsigned)t[3] << 16)), (int)(t[4] | ((unsigned)t[5] << 16)), (int)(t[6] | ((unsigned)t[7] << 16)));
+      }
+    }
+    *(int4 *)&dst[r][kc] = v;
+  }
+};
+template <> struct TileLoad<float> {
+  // 64 rows x 32 k of f32 = 256 threads x 8 values (two float4)
+  static __device__ __forceinline__ void load(const float *base, int ld, int row0, int rows_end, int k0, int K, int vec_ok, int tid, float (*dst)[BK + 4]) {
+    const int r = tid >> 2, kc = (tid & 3) * 8;
+    const int row = row0 + r;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+    if (row < rows_end) {
+      const float *p = base + (size_t)row * ld + k0 + kc;
+      if (vec_ok && k0 + kc + 8 <= K) { a = *(const float4 *)p; b = *(const float4 *)(p + 4); }
+      else {
+        float t[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = (k0 + kc + j < K) ? p[j] : 0.f;
+        a = make_float4(t[0], t[1], t[2], t[3]); b = make_float4(t[4], t[5], t[6], t[7]);
+      }
+    }
+    *(float4 *)&dst[r][kc] = a;
+    *(float4 *)&dst[r][kc + 4] = b;
+  }
+};
+
+__global__ void __launch_bounds__(256) gemm_tile_bf16_kernel(GemmArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t As[BM][BK + 8];
+  __shared__ __attribute__((aligned(16))) uint16_t Ws[BN][BK + 8];
+  int row_lo = 0, row_hi = a.M;
+  const bf16_t *W = (const bf16_t *)a.W;
+  if (a.bounds) {
+    row_lo = a.bounds[blockIdx.z];
+    row_hi = a.bounds[blockIdx.z + 1];
+    W += (size_t)blockIdx.z * a.wstride;
+  }
+  const int m0 = row_lo + blockIdx.y * BM, n0 = blockIdx.x * BN;
+  if (m0 >= row_hi) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ql = lane & 31, kh = lane >> 5;
+  const int wm = (wave & 1) * 32, wn = (wave >> 1) * 32;
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+    TileLoad<bf16_t>::load((const bf16_t *)a.A, a.lda, m0, row_hi, k0, a.K, a.vec_ok, tid, As);
+    TileLoad<bf16_t>::load(W, a.ldw, n0, a.N, k0, a.K, a.vec_ok, tid, Ws);
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 16) {
+      const bf16x8 af = __builtin_bit_cast(bf16x8, *(const int4 *)&As[wm + ql][ks + 8 * kh]);
+      const bf16x8 wf = __builtin_bit_cast(bf16x8, *(const int4 *)&Ws[wn + ql][ks + 8 * kh]);
+      // D[i][j] = sum_k X[i][k] Y[k][j]: X = weights (i = output column n), Y = activations (j = row m): a lane then holds 16 n for ONE m... the other way round
+      // keeps stores coalesced: X = activations (i = m), Y = weights (j = n); lane (ql, kh) ends up with column n = ql and rows (r & 3) + 8 (r >> 2) + 4 kh
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, wf, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const int n = n0 + wn + ql;
+  if (n < a.N) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = m0 + wm + (r & 3) + 8 * (r >> 2) + 4 * kh;
+      if (m < row_hi) {
+        float *c = a.C + (size_t)m * a.ldc + n;
+        *c = a.accumulate ? *c + acc[r] : acc[r];
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
+  __shared__ __attribute__((aligned(16))) float As[BM][BK + 4];
+  __shared__ __attribute__((aligned(16))) float Ws[BN][BK + 4];
+  int row_lo = 0, row_hi = a.M;
+  const float *W = (const float *)a.W;
+  if (a.bounds) {
+    row_lo = a.bounds[blockIdx.z];
+    row_hi = a.bounds[blockIdx.z + 1];
+    W += (size_t)blockIdx.z * a.wstride;
+  }
+  const int m0 = row_lo + blockIdx.y * BM, n0 = blockIdx.x * BN;
+  if (m0 >= row_hi) return;
+  const int tid = threadIdx.x, tn = tid & 15, tm = tid >> 4;  // thread: rows tm + 16 i, columns tn + 16 j
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+    TileLoad<float>::load((const float *)a.A, a.lda, m0, row_hi, k0, a.K, a.vec_ok, tid, As);
+    TileLoad<float>::load(W, a.ldw, n0, a.N, k0, a.K, a.vec_ok, tid, Ws);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; k += 4) {
+      float4 x[4], y[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = *(const float4 *)&As[tm + 16 * i][k];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) y[j] = *(const float4 *)&Ws[tn + 16 * j][k];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] = fmaf(x[i].x, y[j].x, acc[i][j]);
+          acc[i][j] = fmaf(x[i].y, y[j].y, acc[i][j]);
+          acc[i][j] = fmaf(x[i].z, y[j].z, acc[i][j]);
+          acc[i][j] = fmaf(x[i].w, y[j].w, acc[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + tm + 16 * i;
+    if (m >= row_hi) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tn + 16 * j;
+      if (n < a.N) {
+        float *c = a.C + (size_t)m * a.ldc + n;
+        *c = a.accumulate ? *c + acc[i][j] : acc[i][j];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------- M <= 8 rows
+struct GemvArgs {
+  const void *A;
+  const void *W;
+  float *C;
+  int M, N, K, lda, ldw, ldc;
+  int accumulate;
+  const int *row_group;      // grouped: row m multiplies W + row_group[m] * wstride (grid.y = M, one row per workgroup row), else null
+  long long wstride;
+  int vec_ok;
+};
+
+template <class T> struct Vec8;
+template <> struct Vec8<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t *p, float *o) {
+    const int4 v = *(const int4 *)p;
+    const unsigned u[4] = {(unsigned)v.x, (unsigned)v.y, (unsigned)v.z, (unsigned)v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { o[2 * j] = __uint_as_float(u[j] << 16); o[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u); }
+  }
+  static __device__ __forceinline__ void load_nt(const bf16_t *p, float *o) {
+    const int4 v = ld16nt_a4(p);
+    const unsigned u[4] = {(unsigned)v.x, (unsigned)v.y, (unsigned)v.z, (unsigned)v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { o[2 * j] = __uint_as_float(u[j] << 16); o[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u); }
+  }
+};
+template <> struct Vec8<float> {
+  static __device__ __forceinline__ void load(const float *p, float *o) {
+    const float4 a = *(const float4 *)p, b = *(const float4 *)(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+  static __device__ __forceinline__ void load_nt(const float *p, float *o) { load(p, o); }
+};
+
+template <class T, int MR> __global__ void __launch_bounds__(256) gemv_rows_kernel(GemvArgs a) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + wave;
+  if (n >= a.N) return;
+  const T *A = (const T *)a.A;
+  const T *W = (const T *)a.W;
+  int m_lo = 0, m_cnt = a.M;
+  if (a.row_group) {
+    m_lo = blockIdx.y;
+    m_cnt = 1;
+    W += (size_t)a.row_group[m_lo] * a.wstride;
+  }
+  const T *wr = W + (size_t)n * a.ldw;
+  float acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+  if (a.vec_ok) {
+    for (int k = lane * 8; k < a.K; k += 512) {
+      float w[8], x[8];
+      Vec8<T>::load_nt(wr + k, w);
+#pragma unroll
+      for (int m = 0; m < MR; ++m)
+        if (m < m_cnt) {
+          Vec8<T>::load(A + (size_t)(m_lo + m) * a.lda + k, x);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[m] = fmaf(w[j], x[j], acc[m]);
+        }
+    }
+  } else {
+    for (int k = lane; k < a.K; k += 64) {
+      const float w = to_f<T>(wr[k]);
+#pragma unroll
+      for (int m = 0; m < MR; ++m)
+        if (m < m_cnt) acc[m] = fmaf(w, to_f<T>(A[(size_t)(m_lo + m) * a.lda + k]), acc[m]);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    if (m >= m_cnt) break;
+    const float s = wave_sum(acc[m]);
+    if (lane == 0) {
+      float *c = a.C + (size_t)(m_lo + m) * a.ldc + n;
+      *c = a.accumulate ? *c + s : s;
+    }
+  }
+}
+
+static thread_local char g_err[256];
+static int fail(const char *m) { snprintf(g_err, sizeof g_err, "%s", m); return 1; }
+
+}  // namespace hyb
+}  // namespace mrs
+
+using namespace mrs::hyb;
+
+extern "C" const char *mrs_hyb_gemm_last_error() { return g_err; }
+
+// dtype: 1 bf16, 2 f32.  groups > 0: grouped form (bounds [groups + 1] on the device, max_rows = the largest number of rows a group can have).
+extern "C" int mrs_hyb_gemm(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
+                            const int *bounds, int groups, long long wstride, int max_rows, void *stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2)) return fail("mrs_hyb_gemm: bad shape / dtype");
+  const int esz = dtype == 1 ? 2 : 4, vq = 8;
+  GemmArgs a{A, W, C, M, N, K, lda, ldw, ldc, accumulate, groups > 0 ? bounds : nullptr, wstride,
+             (K % vq == 0 && lda % vq == 0 && ldw % vq == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0) ? 1 : 0};
+  const int rows = groups > 0 ? max_rows : M;
+  if (rows <= 0) return 0;
+  dim3 grid((N + BN - 1) / BN, (rows + BM - 1) / BM, groups > 0 ? groups : 1);
+  if (grid.y > 65535 || grid.z > 65535) return fail("mrs_hyb_gemm: too many row tiles / groups for one launch");
+  if (dtype == 1) hipLaunchKernelGGL(gemm_tile_bf16_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(gemm_tile_f32_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemm: launch failed");
+}
+
+extern "C" int mrs_hyb_gemv(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
+                            const int *row_group, long long wstride, void *stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2)) return fail("mrs_hyb_gemv: bad shape / dtype");
+  if (!row_group && M > 8) return fail("mrs_hyb_gemv: at most 8 rows share a weight");
+  if (row_group && M > 65535) return fail("mrs_hyb_gemv: too many rows");
+  const int esz = dtype == 1 ? 2 : 4;
+  GemvArgs a{A, W, C, M, N, K, lda, ldw, ldc, accumulate, row_group, wstride,
+             (K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0) ? 1 : 0};
+  dim3 grid((N + 3) / 4, row_group ? M : 1);
+  hipStream_t s = (hipStream_t)stream;
+#define MRS_GEMV(T, MR) hipLaunchKernelGGL((gemv_rows_kernel<T, MR>), grid, dim3(256), 0, s, a)
+  const int mr = row_group ? 1 : M;
+  if (dtype == 1) { if (mr <= 1) MRS_GEMV(mrs::bf16_t, 1); else if (mr <= 2) MRS_GEMV(mrs::bf16_t, 2); else if (mr <= 4) MRS_GEMV(mrs::bf16_t, 4); else MRS_GEMV(mrs::bf16_t, 8); }
+  else { if (mr <= 1) MRS_GEMV(float, 1); else if (mr <= 2) MRS_GEMV(float, 2); else if (mr <= 4) MRS_GEMV(float, 4); else MRS_GEMV(float, 8); }
+#undef MRS_GEMV
+  return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemv: launch failed");
+}

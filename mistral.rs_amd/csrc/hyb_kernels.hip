@@ -1,0 +1,500 @@
+// hyb_kernels.hip -- the non-GEMM kernels of layer-list ("hybrid") decoders on ragged batches: a step's tokens are ONE flat row range, entry s of the batch owns rows
+// [seq_start[s], seq_start[s + 1]) at positions seq_pos0[s] + i, so prompt portions of any length and single decoded tokens run in the same launches.
+//
+//   embedding gather, RMS norm (plain or one-plus weights; also the per-token 1 / rms for later consumers), grouped RMS norm,
+//   short causal convolution + SiLU with carried taps, the state-space-duality recurrence with a carried f32 state,
+//   whole-projection query / key norm + interleaved partial rotary + paged K / V write, paged attention with a sliding window and kept first tokens,
+//   sigmoid top-k routing, stable expert dispatch, scaled row gather, SiLU-GLU, weighted combine with a gated shared expert.
+//
+// What is f32 regardless of the serving dtype: the residual stream, every norm, positions and angles, scores / softmax / the weighted value sum, router logits and
+// scores, decays, step sizes and the recurrent state.  T below is the dtype of GEMM operands and of the K / V pages: bf16, or f32 in the all-f32 mode.
+#include "common.cuh"
+#include <float.h>
+
+namespace mrs {
+namespace hyb {
+
+static thread_local char g_err[256];
+static int fail(const char *m) { snprintf(g_err, sizeof g_err, "%s", m); return 1; }
+static int ok_or(const char *what) {
+  if (hipGetLastError() == hipSuccess) return 0;
+  snprintf(g_err, sizeof g_err, "%s: launch failed", what);
+  return 1;
+}
+
+__device__ __forceinline__ float block_sum_256(float v, float *red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
+__device__ __forceinline__ float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
+
+// ---------------------------------------------------------------------------------- embedding rows -> f32 residual
+template <class T> __global__ void __launch_bounds__(256) embed_kernel(const int *__restrict__ tokens, const T *__restrict__ table, float *__restrict__ x, int W, int vocab) {
+  const int t = blockIdx.x;
+  int id = tokens[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  for (int c = threadIdx.x; c < W; c += 256) x[(size_t)t * W + c] = to_f<T>(table[(size_t)id * W + c]);
+}
+
+// ---------------------------------------------------------------------------------- x / sqrt(mean(x^2) + eps) * (w | 1 + w); grid.y = equal parts of the row
+template <class T> __global__ void __launch_bounds__(256) rmsnorm_kernel(const float *__restrict__ x, int ldx, const float *__restrict__ w, T *__restrict__ out, float *__restrict__ out32,
+                                                                          float *__restrict__ rstd, int part, float eps, int one_plus, int ldo) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, g = blockIdx.y;
+  const float *xr = x + (size_t)t * ldx + (size_t)g * part;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < part; c += 256) s = fmaf(xr[c], xr[c], s);
+  s = block_sum_256(s, red);
+  const float inv = 1.0f / sqrtf(s / (float)part + eps);
+  if (rstd && threadIdx.x == 0) rstd[(size_t)t * gridDim.y + g] = inv;
+  for (int c = threadIdx.x; c < part; c += 256) {
+    const float wv = w[(size_t)g * part + c];
+    const float v = xr[c] * inv * (one_plus ? 1.0f + wv : wv);
+    if (out) out[(size_t)t * ldo + (size_t)g * part + c] = from_f<T>(v);
+    if (out32) out32[(size_t)t * ldo + (size_t)g * part + c] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------- short causal convolution + SiLU with carried taps
+// u [rows, ldu] (the channels start at column 0 of the pointer handed in), cw [C, taps] (the last column multiplies the current token), state [slots, C, taps - 1]
+// (oldest first).  An entry that starts at position 0 reads zeros instead of its slot.
+__global__ void __launch_bounds__(256) conv_silu_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ cw, const float *__restrict__ cb, const float *__restrict__ state,
+                                                        const int *__restrict__ tok_seq, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
+                                                        const int *__restrict__ seq_slot, float *__restrict__ out, int C, int taps) {
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int s = tok_seq[t], r0 = seq_start[s], i = t - r0;
+  const bool carried = seq_pos0[s] > 0;
+  const float *st = state + ((size_t)seq_slot[s] * C + c) * (taps - 1);
+  float acc = cb[c];
+  for (int j = 0; j < taps; ++j) {
+    const int idx = i - (taps - 1) + j;
+    float v = 0.f;
+    if (idx >= 0) v = u[(size_t)(r0 + idx) * ldu + c];
+    else if (carried) v = st[(taps - 1) + idx];
+    acc = fmaf(cw[(size_t)c * taps + j], v, acc);
+  }
+  out[(size_t)t * C + c] = silu_f(acc);
+}
+// the slot's taps after the step: the last taps - 1 inputs of (old taps ++ this step's rows).  One thread per (entry, channel) reads everything before it writes.
+__global__ void __launch_bounds__(256) conv_state_kernel(const float *__restrict__ u, int ldu, float *__restrict__ state, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
+                                                         const int *__restrict__ seq_slot, int C, int taps) {
+  const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int r0 = seq_start[s], len = seq_start[s + 1] - r0, keep = taps - 1;
+  if (len <= 0) return;
+  const bool carried = seq_pos0[s] > 0;
+  float *st = state + ((size_t)seq_slot[s] * C + c) * keep;
+  float v[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    if (k >= keep) break;
+    const int idx = len - keep + k;
+    v[k] = idx >= 0 ? u[(size_t)(r0 + idx) * ldu + c] : (carried ? st[keep + idx] : 0.f);
+  }
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    if (k >= keep) break;
+    st[k] = v[k];
+  }
+}
+
+// ---------------------------------------------------------------------------------- state-space-duality recurrence, token by token, f32 state carried in a slot
+//   dt = softplus(dt_raw + dt_bias_h);  S <- exp(-exp(A_log_h) dt) S + dt B x^T  (S: N x P);  y = S^T C + D_h x;  out = y * silu(z)
+// One wave per (entry, head, tile of P): lane = (p, r), r in [0, R) owns the state rows n = r + R k; the sum over n closes with R-lane butterflies.  No LDS, no barrier: the
+// per-token chain is the FMA pass plus log2(R) shuffles, and the next token's operands are requested before the current one is used.
+struct ScanArgs {
+  const float *xbc;   // [rows, C]: x [heads * P] | B [G * N] | C [G * N] after convolution + SiLU
+  const float *u;     // [rows, ldu] projection: z at column 0, dt_raw at column dt_col
+  const float *dt_bias, *A_log, *D;
+  float *state;       // [slots, heads, N, P]
+  float *out;         // [rows, heads * P]
+  const int *seq_start, *seq_pos0, *seq_slot;
+  int C, ldu, dt_col, heads, P, N, G;
+};
+template <int R, int MAXK> __global__ void __launch_bounds__(64) ssd_scan_kernel(ScanArgs a) {
+  constexpr int PT = 64 / R;
+  const int lane = threadIdx.x, r = lane % R, p = blockIdx.x * PT + lane / R;
+  const int h = blockIdx.y, s = blockIdx.z;
+  const int r0 = a.seq_start[s], len = a.seq_start[s + 1] - r0;
+  if (len <= 0) return;
+  const bool live = p < a.P;
+  const int pc = live ? p : a.P - 1;
+  const int g = h / (a.heads / a.G), inner = a.heads * a.P;
+  const int nk = (a.N - r + R - 1) / R;  // rows n = r + R k < N
+  float *st = a.state + (((size_t)a.seq_slot[s] * a.heads + h) * a.N) * a.P;
+  float S[MAXK];
+#pragma unroll
+  for (int k = 0; k < MAXK; ++k) S[k] = (k < nk && a.seq_pos0[s] > 0) ? st[(size_t)(r + R * k) * a.P + pc] : 0.f;
+  const float Ah = -expf(a.A_log[h]), Dh = a.D[h], bias = a.dt_bias[h];
+  const int bcol = inner + g * a.N, ccol = inner + a.G * a.N + g * a.N;
+  float Bc[MAXK], Cc[MAXK], Bn[MAXK], Cn[MAXK], xv, dtr, zv, xv_n = 0.f, dtr_n = 0.f, zv_n = 0.f;
+  auto request = [&](int row, float *B_, float *C_, float &x_, float &d_, float &z_) {
+    const float *xr = a.xbc + (size_t)row * a.C;
+#pragma unroll
+    for (int k = 0; k < MAXK; ++k) {
+      const int n = r + R * k;
+      B_[k] = k < nk ? xr[bcol + n] : 0.f;
+      C_[k] = k < nk ? xr[ccol + n] : 0.f;
+    }
+    x_ = xr[h * a.P + pc];
+    d_ = a.u[(size_t)row * a.ldu + a.dt_col + h];
+    z_ = a.u[(size_t)row * a.ldu + h * a.P + pc];
+  };
+  request(r0, Bc, Cc, xv, dtr, zv);
+  for (int i = 0; i < len; ++i) {
+    if (i + 1 < len) request(r0 + i + 1, Bn, Cn, xv_n, dtr_n, zv_n);
+    const float dt = softplus_f(dtr + bias);
+    const float decay = expf(Ah * dt), dx = dt * xv;
+    float part = 0.f;
+#pragma unroll
+    for (int k = 0; k < MAXK; ++k) {
+      S[k] = fmaf(decay, S[k], dx * Bc[k]);
+      part = fmaf(S[k], Cc[k], part);
+    }
+#pragma unroll
+    for (int m = 1; m < R; m <<= 1) part += __shfl_xor(part, m, 64);
+    if (r == 0 && live) a.out[(size_t)(r0 + i) * inner + h * a.P + p] = fmaf(Dh, xv, part) * silu_f(zv);
+#pragma unroll
+    for (int k = 0; k < MAXK; ++k) { Bc[k] = Bn[k]; Cc[k] = Cn[k]; }
+    xv = xv_n; dtr = dtr_n; zv = zv_n;
+  }
+  if (live)
+#pragma unroll
+    for (int k = 0; k < MAXK; ++k)
+      if (k < nk) st[(size_t)(r + R * k) * a.P + p] = S[k];
+}
+
+// ---------------------------------------------------------------------------------- query / key norm over the whole projection, partial interleaved rotary, K / V page write
+struct QkArgs {
+  const float *qkv;   // [rows, ld]: q [H * D] | k [G * D] | v [G * Dv]
+  const float *qw, *kw;  // plain norm weights over the whole projection (null: no norm)
+  const float *freq;  // [rot / 2] angular frequencies
+  const int *tok_pos;
+  const long long *slot_mapping;  // [rows] page slot = block * block_size + offset
+  void *q_out;        // [rows, H * D] in T
+  void *k_cache, *v_cache;  // [blocks, G, block_size, D | Dv] in T
+  int ld, H, G, D, Dv, rot, block_size;
+  float eps;
+};
+template <class T> __global__ void __launch_bounds__(256) qk_norm_rope_cache_kernel(QkArgs a) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int nq = a.H * a.D, nk = a.G * a.D, nv = a.G * a.Dv;
+  const float *q = a.qkv + (size_t)t * a.ld, *k = q + nq, *v = k + nk;
+  float iq = 1.f, ik = 1.f;
+  if (a.qw) {
+    float s = 0.f;
+    for (int c = tid; c < nq; c += 256) s = fmaf(q[c], q[c], s);
+    iq = 1.0f / sqrtf(block_sum_256(s, red) / (float)nq + a.eps);
+  }
+  if (a.kw) {
+    float s = 0.f;
+    for (int c = tid; c < nk; c += 256) s = fmaf(k[c], k[c], s);
+    ik = 1.0f / sqrtf(block_sum_256(s, red) / (float)nk + a.eps);
+  }
+  const float pos = (float)a.tok_pos[t];
+  const long long slot = a.slot_mapping[t];
+  const long long blk = slot / a.block_size;
+  const int off = (int)(slot % a.block_size);
+  T *qo = (T *)a.q_out + (size_t)t * nq;
+  for (int e2 = tid; e2 < (nq + nk) / 2; e2 += 256) {
+    const bool is_q = e2 < nq / 2;
+    const int e = is_q ? 2 * e2 : 2 * e2 - nq;
+    const float *src = is_q ? q : k;
+    const float inv = is_q ? iq : ik;
+    const float *w = is_q ? a.qw : a.kw;
+    float x0 = src[e] * inv, x1 = src[e + 1] * inv;
+    if (w) { x0 *= w[e]; x1 *= w[e + 1]; }
+    const int d = e % a.D;
+    if (d < a.rot) {
+      float sn, cs;
+      sincosf(pos * a.freq[d >> 1], &sn, &cs);
+      const float y0 = x0 * cs - x1 * sn, y1 = x1 * cs + x0 * sn;
+      x0 = y0; x1 = y1;
+    }
+    if (is_q) { qo[e] = from_f<T>(x0); qo[e + 1] = from_f<T>(x1); }
+    else if (slot >= 0) {
+      const int g = e / a.D;
+      T *kc = (T *)a.k_cache + (((size_t)blk * a.G + g) * a.block_size + off) * a.D + d;
+      kc[0] = from_f<T>(x0); kc[1] = from_f<T>(x1);
+    }
+  }
+  if (slot >= 0)
+    for (int e = tid; e < nv; e += 256) {
+      const int g = e / a.Dv, d = e % a.Dv;
+      ((T *)a.v_cache)[(((size_t)blk * a.G + g) * a.block_size + off) * a.Dv + d] = from_f<T>(v[e]);
+    }
+}
+
+// ---------------------------------------------------------------------------------- paged attention, sliding window with kept first tokens
+// Query at position i sees key j <= i when i - j < window or j < keep_first (window <= 0: every j <= i).  One wave per (row, head): keys in passes of 64 (a lane = a key for the
+// scores, a lane = value dimensions for the weighted sum), running maximum / sum in f32.
+struct AttnArgs {
+  const void *q;        // [rows, H * D] in T
+  const void *k_cache, *v_cache;
+  const int *block_tables;  // [entries, max_blocks]
+  const int *tok_seq, *tok_pos;
+  void *out;            // [rows, H * Dv] in T
+  int H, G, D, Dv, block_size, max_blocks, window, keep_first;
+  float scale;
+};
+template <class T, int DVC> __global__ void __launch_bounds__(64) paged_window_attn_kernel(AttnArgs a) {
+  extern __shared__ float lds[];  // q [D] | p [64] | key row index [64] as int
+  float *qs = lds, *ps = lds + a.D;
+  long long *rowbase = (long long *)(ps + 64 + ((a.D & 1) ? 1 : 0));
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int s = a.tok_seq[t], i = a.tok_pos[t], g = h / (a.H / a.G);
+  const T *q = (const T *)a.q + ((size_t)t * a.H + h) * a.D;
+  for (int d = lane; d < a.D; d += 64) qs[d] = to_f<T>(q[d]);
+  const int *bt = a.block_tables + (size_t)s * a.max_blocks;
+  int w_lo = a.window > 0 ? i - a.window + 1 : 0;
+  if (w_lo < 0) w_lo = 0;
+  int n1 = a.keep_first < w_lo ? a.keep_first : w_lo;  // kept first tokens that the window does not already cover
+  if (n1 < 0) n1 = 0;
+  const int total = n1 + (i - w_lo + 1);
+  float m = -FLT_MAX, l = 0.f, o[DVC];
+#pragma unroll
+  for (int c = 0; c < DVC; ++c) o[c] = 0.f;
+  MRS_WAVE_SYNC();
+  for (int v0 = 0; v0 < total; v0 += 64) {
+    const int vi = v0 + lane;
+    float sc = -FLT_MAX;
+    long long base = -1;
+    if (vi < total) {
+      const int key = vi < n1 ? vi : w_lo + (vi - n1);
+      base = ((long long)bt[key / a.block_size] * a.G + g) * a.block_size + key % a.block_size;
+      const T *kr = (const T *)a.k_cache + (size_t)base * a.D;
+      float acc = 0.f;
+      for (int d = 0; d < a.D; ++d) acc = fmaf(qs[d], to_f<T>(kr[d]), acc);
+      sc = acc * a.scale;
+    }
+    const float mn = fmaxf(m, wave_max(sc));
+    const float alpha = expf(m - mn);
+    const float p = vi < total ? expf(sc - mn) : 0.f;
+    l = l * alpha + wave_sum(p);
+    m = mn;
+    MRS_WAVE_SYNC();
+    ps[lane] = p;
+    rowbase[lane] = base;
+    MRS_WAVE_SYNC();
+    const int cnt = total - v0 < 64 ? total - v0 : 64;
+#pragma unroll
+    for (int c = 0; c < DVC; ++c) {
+      const int d = lane + 64 * c;
+      float acc = o[c] * alpha;
+      if (d < a.Dv)
+        for (int j = 0; j < cnt; ++j) acc = fmaf(ps[j], to_f<T>(((const T *)a.v_cache)[(size_t)rowbase[j] * a.Dv + d]), acc);
+      o[c] = acc;
+    }
+  }
+  const float inv = 1.0f / l;
+  T *out = (T *)a.out + ((size_t)t * a.H + h) * a.Dv;
+#pragma unroll
+  for (int c = 0; c < DVC; ++c) {
+    const int d = lane + 64 * c;
+    if (d < a.Dv) out[d] = from_f<T>(o[c] * inv);
+  }
+}
+
+// ---------------------------------------------------------------------------------- mixture of experts: routing, dispatch, gather, GLU, combine
+// z [rows, ldz]: E router logits (+ the shared expert's gate logit at column E when has_gate).  score = sigmoid(z); the `top` largest (ties: the lower index), weights = scores.
+__global__ void __launch_bounds__(256) route_sigmoid_topk_kernel(const float *__restrict__ z, int ldz, int rows, int E, int top, int has_gate, int *__restrict__ ids,
+                                                                 float *__restrict__ wts, float *__restrict__ gate) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= rows) return;
+  const float *zr = z + (size_t)t * ldz;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = -FLT_MAX;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken |= ids[(size_t)t * top + j] == e;
+      if (!taken && (best < 0 || zr[e] > bv)) { best = e; bv = zr[e]; }
+    }
+    ids[(size_t)t * top + k] = best;
+    wts[(size_t)t * top + k] = sigmoid_f(bv);
+  }
+  if (has_gate) gate[t] = sigmoid_f(zr[E]);
+}
+// stable counting sort of the routes by expert: bounds [E + 1], sorted_route [R] (route index = token * top + k), route_pos [R] (its inverse), sorted_expert [R]
+__global__ void __launch_bounds__(1024) moe_dispatch_kernel(const int *__restrict__ ids, int R, int E, int *__restrict__ bounds, int *__restrict__ sorted_route,
+                                                           int *__restrict__ route_pos, int *__restrict__ sorted_expert) {
+  extern __shared__ int cnt[];  // [E + 1]
+  for (int e = threadIdx.x; e < E; e += 1024) {
+    int c = 0;
+    for (int r = 0; r < R; ++r) c += ids[r] == e;
+    cnt[e] = c;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) { const int c = cnt[e]; cnt[e] = run; bounds[e] = run; run += c; }
+    bounds[E] = run;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 1024) {
+    int at = cnt[e];
+    for (int r = 0; r < R; ++r)
+      if (ids[r] == e) { sorted_route[at] = r; route_pos[r] = at; sorted_expert[at] = e; ++at; }
+  }
+}
+// row i of the expert-sorted operand = weight of its route * the token's normed row (f32), rounded once to T
+template <class T> __global__ void __launch_bounds__(256) moe_gather_kernel(const float *__restrict__ h32, const int *__restrict__ sorted_route, const float *__restrict__ wts, int top,
+                                                                            T *__restrict__ out, int W) {
+  const int i = blockIdx.x, r = sorted_route[i], t = r / top;
+  const float w = wts[r];
+  for (int c = threadIdx.x; c < W; c += 256) out[(size_t)i * W + c] = from_f<T>(w * h32[(size_t)t * W + c]);
+}
+// silu(gate) * up; gu [rows, 2 ff] = gate | up
+template <class T> __global__ void __launch_bounds__(256) glu_silu_kernel(const float *__restrict__ gu, T *__restrict__ out, int rows, int ff) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)rows * ff) return;
+  const size_t r = i / ff, c = i % ff;
+  const float gv = gu[r * 2 * ff + c], uv = gu[r * 2 * ff + ff + c];
+  out[i] = from_f<T>(silu_f(gv) * uv);
+}
+// x[t] += sum_k d[route_pos[t top + k]] + gate[t] * shared[t]
+__global__ void __launch_bounds__(256) moe_combine_kernel(float *__restrict__ x, const float *__restrict__ d, const int *__restrict__ route_pos, int top, const float *__restrict__ shared,
+                                                          const float *__restrict__ gate, int W) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) acc += d[(size_t)route_pos[(size_t)t * top + k] * W + c];
+    if (shared) acc += (gate ? gate[t] : 1.0f) * shared[(size_t)t * W + c];
+    x[(size_t)t * W + c] += acc;
+  }
+}
+__global__ void __launch_bounds__(256) gather_rows_kernel(const float *__restrict__ x, const int *__restrict__ idx, float *__restrict__ out, int W) {
+  const int i = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += 256) out[(size_t)i * W + c] = x[(size_t)idx[i] * W + c];
+}
+
+}  // namespace hyb
+}  // namespace mrs
+
+using namespace mrs::hyb;
+#define S_(s) ((hipStream_t)(s))
+
+extern "C" const char *mrs_hyb_last_error() { return g_err; }
+
+extern "C" int mrs_hyb_embed(const int *tokens, const void *table, float *x, int rows, int W, int vocab, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  if (dtype == 1) hipLaunchKernelGGL(embed_kernel<mrs::bf16_t>, dim3(rows), dim3(256), 0, S_(stream), tokens, (const mrs::bf16_t *)table, x, W, vocab);
+  else if (dtype == 2) hipLaunchKernelGGL(embed_kernel<float>, dim3(rows), dim3(256), 0, S_(stream), tokens, (const float *)table, x, W, vocab);
+  else return fail("mrs_hyb_embed: dtype");
+  return ok_or("mrs_hyb_embed");
+}
+
+// parts > 1: every row is normed in `parts` equal pieces, each by its own root mean square.  out (dtype) and / or out32 (f32) receive the result, rstd [rows, parts] the 1 / rms.
+extern "C" int mrs_hyb_rmsnorm(const float *x, int ldx, const float *w, void *out, float *out32, float *rstd, int rows, int width, int parts, float eps, int one_plus, int dtype,
+                               void *stream) {
+  if (rows <= 0) return 0;
+  if (parts <= 0 || width % parts) return fail("mrs_hyb_rmsnorm: the row does not split into equal parts");
+  dim3 grid(rows, parts);
+  if (dtype == 1) hipLaunchKernelGGL(rmsnorm_kernel<mrs::bf16_t>, grid, dim3(256), 0, S_(stream), x, ldx, w, (mrs::bf16_t *)out, out32, rstd, width / parts, eps, one_plus, width);
+  else if (dtype == 2) hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, dim3(256), 0, S_(stream), x, ldx, w, (float *)out, out32, rstd, width / parts, eps, one_plus, width);
+  else return fail("mrs_hyb_rmsnorm: dtype");
+  return ok_or("mrs_hyb_rmsnorm");
+}
+
+extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const float *cb, float *state, const int *tok_seq, const int *seq_start, const int *seq_pos0,
+                                 const int *seq_slot, float *out, int rows, int entries, int C, int taps, void *stream) {
+  if (rows <= 0) return 0;
+  if (taps < 1 || taps > 17) return fail("mrs_hyb_conv_silu: 1 .. 17 taps");
+  hipLaunchKernelGGL(conv_silu_kernel, dim3(rows, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps);
+  if (taps > 1)
+    hipLaunchKernelGGL(conv_state_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, state, seq_start, seq_pos0, seq_slot, C, taps);
+  return ok_or("mrs_hyb_conv_silu");
+}
+
+extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, float *state, float *out, const int *seq_start,
+                                const int *seq_pos0, const int *seq_slot, int entries, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream) {
+  if (entries <= 0) return 0;
+  if (heads <= 0 || G <= 0 || heads % G || P <= 0 || N <= 0) return fail("mrs_hyb_ssd_scan: bad head / group sizes");
+  ScanArgs a{xbc, u, dt_bias, A_log, D, state, out, seq_start, seq_pos0, seq_slot, C, ldu, dt_col, heads, P, N, G};
+#define MRS_SCAN(R, K) hipLaunchKernelGGL((ssd_scan_kernel<R, K>), dim3((P + 64 / R - 1) / (64 / R), heads, entries), dim3(64), 0, S_(stream), a)
+  if (N <= 16) MRS_SCAN(2, 8);
+  else if (N <= 64) MRS_SCAN(4, 16);
+  else if (N <= 128) MRS_SCAN(4, 32);
+  else if (N <= 256) MRS_SCAN(8, 32);
+  else if (N <= 512) MRS_SCAN(16, 32);
+  else return fail("mrs_hyb_ssd_scan: state size above 512");
+#undef MRS_SCAN
+  return ok_or("mrs_hyb_ssd_scan");
+}
+
+extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping,
+                                          void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int rot, int block_size, float eps, int dtype,
+                                          void *stream) {
+  if (rows <= 0) return 0;
+  if ((D & 1) || (rot & 1) || rot > D || rot < 0 || H <= 0 || G <= 0 || H % G) return fail("mrs_hyb_qk_norm_rope_cache: head sizes (even dim, even rot <= dim, heads % kv_heads == 0)");
+  QkArgs a{qkv, qw, kw, freq, tok_pos, slot_mapping, q_out, k_cache, v_cache, ld, H, G, D, Dv, rot, block_size, eps};
+  if (dtype == 1) hipLaunchKernelGGL(qk_norm_rope_cache_kernel<mrs::bf16_t>, dim3(rows), dim3(256), 0, S_(stream), a);
+  else if (dtype == 2) hipLaunchKernelGGL(qk_norm_rope_cache_kernel<float>, dim3(rows), dim3(256), 0, S_(stream), a);
+  else return fail("mrs_hyb_qk_norm_rope_cache: dtype");
+  return ok_or("mrs_hyb_qk_norm_rope_cache");
+}
+
+extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
+                                         int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  if (Dv > 256 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 256 / heads % kv_heads");
+  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale};
+  const size_t lds = (size_t)(D + 64 + 2) * 4 + 64 * 8;
+  dim3 grid(rows, H);
+#define MRS_ATTN(T, C) hipLaunchKernelGGL((paged_window_attn_kernel<T, C>), grid, dim3(64), lds, S_(stream), a)
+  const int c = (Dv + 63) / 64;
+  if (dtype == 1) { if (c <= 1) MRS_ATTN(mrs::bf16_t, 1); else if (c <= 2) MRS_ATTN(mrs::bf16_t, 2); else MRS_ATTN(mrs::bf16_t, 4); }
+  else if (dtype == 2) { if (c <= 1) MRS_ATTN(float, 1); else if (c <= 2) MRS_ATTN(float, 2); else MRS_ATTN(float, 4); }
+  else return fail("mrs_hyb_paged_window_attn: dtype");
+#undef MRS_ATTN
+  return ok_or("mrs_hyb_paged_window_attn");
+}
+
+extern "C" int mrs_hyb_route_sigmoid_topk(const float *z, int ldz, int rows, int E, int top, int has_gate, int *ids, float *wts, float *gate, void *stream) {
+  if (rows <= 0) return 0;
+  if (top < 1 || top > E) return fail("mrs_hyb_route_sigmoid_topk: 1 <= top <= experts");
+  hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3((rows + 255) / 256), dim3(256), 0, S_(stream), z, ldz, rows, E, top, has_gate, ids, wts, gate);
+  return ok_or("mrs_hyb_route_sigmoid_topk");
+}
+
+extern "C" int mrs_hyb_moe_dispatch(const int *ids, int R, int E, int *bounds, int *sorted_route, int *route_pos, int *sorted_expert, void *stream) {
+  if (E <= 0 || E > 8192) return fail("mrs_hyb_moe_dispatch: 1 .. 8192 experts");
+  hipLaunchKernelGGL(moe_dispatch_kernel, dim3(1), dim3(1024), (size_t)(E + 1) * 4, S_(stream), ids, R, E, bounds, sorted_route, route_pos, sorted_expert);
+  return ok_or("mrs_hyb_moe_dispatch");
+}
+
+extern "C" int mrs_hyb_moe_gather(const float *h32, const int *sorted_route, const float *wts, int top, void *out, int R, int W, int dtype, void *stream) {
+  if (R <= 0) return 0;
+  if (dtype == 1) hipLaunchKernelGGL(moe_gather_kernel<mrs::bf16_t>, dim3(R), dim3(256), 0, S_(stream), h32, sorted_route, wts, top, (mrs::bf16_t *)out, W);
+  else if (dtype == 2) hipLaunchKernelGGL(moe_gather_kernel<float>, dim3(R), dim3(256), 0, S_(stream), h32, sorted_route, wts, top, (float *)out, W);
+  else return fail("mrs_hyb_moe_gather: dtype");
+  return ok_or("mrs_hyb_moe_gather");
+}
+
+extern "C" int mrs_hyb_glu_silu(const float *gu, void *out, int rows, int ff, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  const unsigned blocks = (unsigned)(((size_t)rows * ff + 255) / 256);
+  if (dtype == 1) hipLaunchKernelGGL(glu_silu_kernel<mrs::bf16_t>, dim3(blocks), dim3(256), 0, S_(stream), gu, (mrs::bf16_t *)out, rows, ff);
+  else if (dtype == 2) hipLaunchKernelGGL(glu_silu_kernel<float>, dim3(blocks), dim3(256), 0, S_(stream), gu, (float *)out, rows, ff);
+  else return fail("mrs_hyb_glu_silu: dtype");
+  return ok_or("mrs_hyb_glu_silu");
+}
+
+extern "C" int mrs_hyb_moe_combine(float *x, const float *d, const int *route_pos, int top, const float *shared, const float *gate, int rows, int W, void *stream) {
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(rows), dim3(256), 0, S_(stream), x, d, route_pos, top, shared, gate, W);
+  return ok_or("mrs_hyb_moe_combine");
+}
+
+extern "C" int mrs_hyb_gather_rows(const float *x, const int *idx, float *out, int n, int W, void *stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, S_(stream), x, idx, out, W);
+  return ok_or("mrs_hyb_gather_rows");
+}

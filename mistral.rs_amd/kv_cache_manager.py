@@ -20,7 +20,7 @@ _P, _SZ, _U64, _I64 = C.c_void_p, C.c_size_t, C.c_uint64, C.c_int64
 
 
 def _f(name, argtypes, restype=None):
-    return _lib.sym("ext", name, argtypes, restype)
+    return _lib.sym(_lib.host_key(), name, argtypes, restype)
 
 
 def _arr(ctype, values):
@@ -165,9 +165,12 @@ class KVCacheManager:
         self._block_size = block_size
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            _f("mrs_kv_manager_destroy", [_P])(self._h)
-            self._h = None
+        try:
+            if getattr(self, "_h", None):
+                _f("mrs_kv_manager_destroy", [_P])(self._h)
+                self._h = None
+        except Exception:  # interpreter shutdown: the loader module may be gone already
+            pass
 
     def block_pool(self) -> BlockPool:
         p = BlockPool(0, False, 0, _borrowed=_f("mrs_kv_manager_pool", [_P], _P)(self._h))
@@ -249,3 +252,39 @@ class KVCacheManager:
         out = (C.c_int32 * max(max_blocks, 1))()
         r = _f("mrs_kv_get_block_table", [_P, _U64, _SZ, _P], C.c_int)(self._h, request_id, max_blocks, out)
         return None if r != 0 else list(out[:max_blocks])
+
+
+class StateSlotPool:
+    """Fixed-size per-sequence state slots (csrc/host/state_pool.cpp): what recurrent mixers carry per live sequence next to the paged K / V blocks.  `allocate` gives the
+    request its slot (the same one on every later call) or None when all are taken -- role of `RecurrentStatePool::allocate / free / num_free_slots`
+    (mistralrs-core/src/kv_cache/hybrid_cache.rs:237-256, 404)."""
+
+    def __init__(self, num_slots: int):
+        self._h = _f("mrs_state_pool_create", [_SZ], _P)(num_slots)
+        if not self._h:
+            raise ValueError("StateSlotPool: needs at least one slot")
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                _f("mrs_state_pool_destroy", [_P])(self._h)
+                self._h = None
+        except Exception:  # interpreter shutdown: the loader module may be gone already
+            pass
+
+    def capacity(self) -> int:
+        return _f("mrs_state_pool_capacity", [_P], _SZ)(self._h)
+
+    def num_free_slots(self) -> int:
+        return _f("mrs_state_pool_num_free_slots", [_P], _SZ)(self._h)
+
+    def allocate(self, request_id: int) -> Optional[int]:
+        r = _f("mrs_state_pool_allocate", [_P, _U64], _I64)(self._h, request_id)
+        return None if r < 0 else r
+
+    def slot_of(self, request_id: int) -> Optional[int]:
+        r = _f("mrs_state_pool_slot_of", [_P, _U64], _I64)(self._h, request_id)
+        return None if r < 0 else r
+
+    def free(self, request_id: int) -> None:
+        _f("mrs_state_pool_free", [_P, _U64])(self._h, request_id)
