@@ -46,6 +46,7 @@ def main(argv=None) -> int:
     os.makedirs(a.out, exist_ok=True)
     ids: dict = {}
     length: dict = {}
+    admitted = 0
     with torch.inference_mode():
         for line in sys.stdin:
             line = line.strip()
@@ -56,7 +57,10 @@ def main(argv=None) -> int:
             for e in step.get("entries", []):
                 if not e["tokens"]:
                     continue
-                rid = ids.setdefault(e["id"], len(ids) + 1)
+                if e["id"] not in ids:
+                    admitted += 1
+                    ids[e["id"]] = admitted
+                rid = ids[e["id"]]
                 p0 = length.get(rid, 0)
                 if not cache.reserve(rid, p0 + len(e["tokens"])):
                     print(f"trace_run: no pages or state slot left for request {e['id']!r}", file=sys.stderr)
