@@ -133,6 +133,25 @@ def sample(packed: np.ndarray, k: int, temperature: float, top_p: float, min_p: 
     return int(ids[j]), float(rep[j])
 
 
+class SequenceSampler:
+    """One sampling configuration applied to logits rows of any model (the engine's `sampler`): top_k == 1 is the arg-max through the top-1 kernels (probability 1),
+    otherwise the device top-k, then the top-p / min-p cuts and the draw on the host (`Sampler::sample` with top_k set, sampler.rs:1262-1290)."""
+
+    def __init__(self, vocab: int, device, top_k: int = 1, temperature: float = 1.0, top_p: float = 1.0, min_p: float = 0.0, seed: int = 0):
+        self.k = min(int(top_k), int(vocab))
+        self.temperature, self.top_p, self.min_p = float(temperature), float(top_p), float(min_p)
+        self.rng = np.random.default_rng(seed)
+        self._t1 = Top1(vocab, device) if self.k == 1 else None
+        self._tk = None if self.k == 1 else TopK(vocab, self.k, device)
+
+    def __call__(self, logits: torch.Tensor):
+        """logits f32 [vocab] on the device -> (token id, reporting probability)"""
+        row = logits.reshape(1, -1).float().contiguous()
+        if self.k == 1:
+            return top1_token(self._t1(row).cpu().numpy()[0]), 1.0
+        return sample(self._tk(row, self.temperature).cpu().numpy()[0], self._tk.k, self.temperature, self.top_p, self.min_p, self.rng)
+
+
 def generate(model, prompt, max_new_tokens: int, top_k: int, temperature: float = 1.0, top_p: float = 1.0, min_p: float = 0.0, seed: int = 0):
     """Sampled decoding on a `Llama` runner (the loop of `Sampler::sample` with top_k set, sampler.rs:1262-1290): prefill, then per token one decode step, the device
     top-k over the logits row, `2k + 2` floats to the host, the top-p / min-p cuts and the draw there.  top_k == 1 takes the arg-max through the top-1 kernels, no temperature, probability 1

@@ -13,7 +13,14 @@ What is restated (line references into scheduler.rs):
     (`_preempt` :1026-1073: state Waiting, computed tokens 0, full blocks published to the prefix cache, blocks freed, FRONT of the waiting queue), then
     take a round-robin window of the running rows under the token budget (`completion_batch_indices` :303-330);
   * `free_finished_sequence_groups` (:957-1024): finished sequences publish their full blocks and release them.
-Not restated: multimodal features, adapters, speculative staging, recurrent state, packed prefill, scheduler-visible chunk plans, metrics.
+  * recurrent state (hybrid models): with a `state_pool` every admitted sequence also holds one state slot (`RecurrentStatePool::allocate`,
+    kv_cache/hybrid_cache.rs:237-256); a sequence that finds pages but no slot waits like one that finds no pages; preemption and completion give the slot back, and
+    a preempted sequence restarts from position 0 (its recurrent state is gone with the slot).  Prefix caching is off for such models: a cached block holds K / V,
+    not the recurrent state of its last token.
+Not restated: multimodal features, adapters, speculative staging, packed prefill, scheduler-visible chunk plans, metrics.
+
+Models with a ragged step function (`forward_batch`: mistralrs_amd.hybrid.HybridDecoder) take prompt batches of unequal portions and completion batches through the same
+call (`SchedulerConfig.uniform_prompt_batches = False`); the Llama runner keeps uniform prompt batches.
 """
 from __future__ import annotations
 
@@ -71,6 +78,7 @@ class SchedulerConfig:
     max_num_seqs: int
     max_num_batched_tokens: int
     max_decode_steps_before_prefill: int = 4
+    uniform_prompt_batches: bool = True   # requires_uniform_prompt_batch: the Llama runner's prompt launches want equal lengths; a ragged step function does not
 
 
 @dataclass
@@ -84,9 +92,11 @@ class SchedulerOutput:
 
 
 class PagedAttentionScheduler:
-    def __init__(self, config: SchedulerConfig, kv_cache_manager: KVCacheManager, prefix_caching: bool = True):
+    def __init__(self, config: SchedulerConfig, kv_cache_manager: KVCacheManager, prefix_caching: bool = True, state_pool=None):
         assert config.max_num_seqs > 0 and config.max_num_batched_tokens > 0 and config.max_decode_steps_before_prefill > 0
         self.config, self.kv = config, kv_cache_manager
+        self.state_pool = state_pool  # kv_cache_manager.StateSlotPool for models with recurrent layers, else None
+        prefix_caching = prefix_caching and state_pool is None
         self.block_size = kv_cache_manager.block_size()
         self.waiting: deque = deque()
         self.running: deque = deque()
@@ -124,14 +134,29 @@ class PagedAttentionScheduler:
         seq.num_computed_tokens = 0
         if self.prefix_caching_enabled:
             self.kv.cache_blocks(seq.id, self._hashes(seq), computed)
-        self.kv.free(seq.id)
+        self._release(seq.id)
         self.waiting.appendleft(seq)
+
+    def _release(self, seq_id: int) -> None:
+        self.kv.free(seq_id)
+        if self.state_pool is not None:
+            self.state_pool.free(seq_id)
+
+    def _admit(self, seq_id: int, n_tok: int, cached_ids) -> bool:
+        """Pages for the whole prompt and, for models with recurrent layers, a state slot: both or neither."""
+        if self.state_pool is not None and self.state_pool.slot_of(seq_id) is None and self.state_pool.num_free_slots() == 0:
+            return False
+        if self.kv.allocate_slots(seq_id, n_tok, cached_ids) is None:
+            return False
+        if self.state_pool is not None:
+            self.state_pool.allocate(seq_id)
+        return True
 
     def _reject_front_of_waiting(self, reason: str) -> None:
         seq = self.waiting.popleft()
         seq.state, seq.error = FINISHED_IGNORED, reason
         self.waiting_counts.pop(seq.id, None)
-        self.kv.free(seq.id)
+        self._release(seq.id)
 
     def prompt_chunk_size(self, batch: int) -> Optional[int]:  # :136-138
         return max(self.config.max_num_batched_tokens // batch, 1) if batch > 0 else None
@@ -208,7 +233,7 @@ class PagedAttentionScheduler:
             cached_ids = list(hit.block_ids) if hit else []
             n_cached = hit.num_computed_tokens if hit else 0
             cached_ids = cached_ids[: n_cached // self.block_size]
-            ok = self.kv.allocate_slots(seq.id, n_tok, cached_ids) is not None
+            ok = self._admit(seq.id, n_tok, cached_ids)
             if ok:
                 self.waiting_counts.pop(seq.id, None)
             else:
@@ -223,7 +248,7 @@ class PagedAttentionScheduler:
                     self._preempt(victim)
                     self.waiting.appendleft(waiting_seq)
                     scheduled = deque(s for s in scheduled if s.id != victim.id)
-                    if self.kv.allocate_slots(seq.id, n_tok, cached_ids) is not None:
+                    if self._admit(seq.id, n_tok, cached_ids):
                         allocated = True
                         break
                 if not allocated:
@@ -235,7 +260,7 @@ class PagedAttentionScheduler:
             self.running.append(seq)
             scheduled.append(seq)
         if scheduled:
-            batch = self._bucket_and_preempt(scheduled)
+            batch = self._bucket_and_preempt(scheduled) if self.config.uniform_prompt_batches else scheduled
             self.decode_steps_since_prefill = 0
             return SchedulerOutput("prompt", list(batch), [s.prefix_cache_len for s in batch], self.prompt_chunk_size(len(batch)), list(self.preempted_sequence_ids))
         # ---- completion: reserve the next token's slot for every running sequence, FCFS, preempting from the back (:791-850)
@@ -275,7 +300,7 @@ class PagedAttentionScheduler:
             if s.is_finished:
                 if self.prefix_caching_enabled:
                     self.kv.cache_blocks(s.id, self._hashes(s), s.num_computed_tokens)
-                self.kv.free(s.id)
+                self._release(s.id)
                 self.waiting_counts.pop(s.id, None)
             else:
                 keep.append(s)
@@ -287,22 +312,52 @@ class PagedEngine:
     `prompt_chunk_size` tokens through the same kernels (so a preempted and recomputed sequence reproduces its logits bit for bit), block tables and slot
     mappings from the KV cache manager (pipeline/inputs_processor.rs:900-922)."""
 
-    def __init__(self, model, scheduler: PagedAttentionScheduler):
+    def __init__(self, model, scheduler: PagedAttentionScheduler, sampler=None):
         self.m, self.s = model, scheduler
-        self.cfg = model.cfg
+        self.ragged = hasattr(model, "forward_batch")  # a ragged step function: unequal prompt portions and single tokens in one call
+        self.cfg = None if self.ragged else model.cfg
+        self.max_context_len = scheduler.kv.num_gpu_blocks() * scheduler.block_size if self.ragged else model.cfg.max_context_len
+        self.sampler = sampler  # sampler.SequenceSampler (top-k / top-p / min-p on the device + host draw); None = arg-max
         self.steps = {"prompt": 0, "completion": 0, "preemptions": 0}
+        if self.ragged and model.has_recurrent_state and scheduler.state_pool is None:
+            raise ValueError("PagedEngine: a model with recurrent layers needs a scheduler with a state_pool")
 
     def _table(self, seq: Sequence):
         import torch
         return torch.tensor(self.s.kv.get_block_table(seq.id, self.cfg.max_blocks_per_seq), dtype=self.m.block_tables.dtype, device=self.m.device)
 
     def _finish_token(self, seq: Sequence, logits) -> None:
-        tok = int(logits.argmax())
+        tok = int(logits.argmax()) if self.sampler is None else self.sampler(logits)[0]
         seq.last_logits = logits.clone()
         seq.tokens.append(tok)
         seq.generated.append(tok)
-        if len(seq.generated) >= seq.max_new_tokens or len(seq.tokens) >= self.cfg.max_context_len:
+        if len(seq.generated) >= seq.max_new_tokens or len(seq.tokens) >= self.max_context_len:
             seq.state = DONE
+
+    def _ragged_step(self, out: SchedulerOutput) -> None:
+        """One call of the model's ragged step function for the whole scheduled batch: a prompt pass brings every sequence's next portion (the prompt's last token, when it is
+        in the portion, asks for logits), a completion pass one token per sequence."""
+        from .hybrid import RaggedBatch
+        entries, ends = [], []
+        for seq in out.scheduled:
+            a = seq.num_computed_tokens
+            b = min(len(seq), a + (out.prompt_chunk_size or len(seq))) if out.kind == "prompt" else len(seq)
+            if b <= a:
+                continue
+            slot = self.s.state_pool.slot_of(seq.id) if self.s.state_pool is not None else 0
+            entries.append({"tokens": seq.tokens[a:b], "pos0": a, "slot": slot, "blocks": self.s.kv.get_block_ids(seq.id) or [],
+                            "want": [b - a - 1] if b == len(seq) else []})
+            ends.append((seq, b))
+        if not entries:
+            return
+        logits = self.m.forward_batch(RaggedBatch.build(entries, self.s.block_size, self.m.device))
+        row = 0
+        for seq, b in ends:
+            seq.num_computed_tokens = b
+            if b == len(seq):
+                seq.state = RUNNING_COMPLETION
+                self._finish_token(seq, logits[row])
+                row += 1
 
     def _p2p_guard(self) -> None:
         """Tensor parallel: before tokens are handed out, the per-rank error word of the peer-mailbox all-reduce is MAX-reduced over the ranks (Llama.p2p_sync_error);
@@ -314,7 +369,10 @@ class PagedEngine:
     def step(self) -> str:
         out = self.s.schedule()
         self.steps["preemptions"] += len(out.preempted)
-        if out.kind == "prompt":
+        if self.ragged and out.kind in ("prompt", "completion"):
+            self.steps[out.kind] += 1
+            self._ragged_step(out)
+        elif out.kind == "prompt":
             self.steps["prompt"] += 1
             for seq in out.scheduled:
                 a = seq.num_computed_tokens

@@ -72,6 +72,22 @@ def visible(i, j, size, keep_first):
     return j <= i and (i - j < size or j < keep_first)
 
 
+def windowed_attention(q, k, v, scale, size, keep_first, pos_q=None):
+    """q [Tq, H, D], k [Tk, G, D], v [Tk, G, Dv]; key j sits at position j, query row r at pos_q[r] (default r).  Softmax over the visible keys, one (query, head) at a time."""
+    Tq, H, _ = q.shape
+    G, Dv = k.shape[1], v.shape[2]
+    pos_q = list(range(Tq)) if pos_q is None else [int(p) for p in pos_q]
+    out = torch.zeros(Tq, H, Dv, dtype=F)
+    for hh in range(H):
+        g = hh // (H // G)
+        for r, i in enumerate(pos_q):
+            js = [j for j in range(min(i + 1, k.shape[0])) if visible(i, j, size if size > 0 else i + 1, keep_first)]
+            s = (k[js, g] @ q[r, hh]) * scale
+            pr = torch.softmax(s, 0)
+            out[r, hh] = pr @ v[js, g]
+    return out
+
+
 def attention_mixer(h, m, w, p, eps):
     """h [T, width] of ONE sequence from position 0.  m: the mixer's config."""
     T = h.shape[0]
@@ -85,15 +101,7 @@ def attention_mixer(h, m, w, p, eps):
     if rot:
         fr = rope_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
         q, k = rope_interleaved(q, pos, fr), rope_interleaved(k, pos, fr)
-    size, keep = m["mask"]["size"], m["mask"]["keep_first"]
-    out = torch.zeros(T, H, Dv, dtype=F)
-    for hh in range(H):
-        g = hh // (H // G)
-        for i in range(T):
-            js = [j for j in range(i + 1) if visible(i, j, size, keep)]
-            s = torch.stack([(q[i, hh] * k[j, g]).sum() for j in js]) * m["scale"]
-            pr = torch.softmax(s, 0)
-            out[i, hh] = (pr[:, None] * v[js, g]).sum(0)
+    out = windowed_attention(q, k, v, m["scale"], m["mask"]["size"], m["mask"]["keep_first"])
     return out.reshape(T, H * Dv) @ w[p + "o"].T
 
 
