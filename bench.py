@@ -574,6 +574,138 @@ def extra_config(kind, dev, steps=64, warmup=4, prompt_len=512):
     return out
 
 
+HYBRID_SIZES = {
+    # layer lists that resemble a small and a mid-size hybrid mixture-of-experts model: three state-space layers per attention layer
+    "s": dict(width=1024, layers=8, m_heads=32, m_vdim=64, state=128, groups=4, a_heads=16, a_kv=4, dim=128, vdim=128, window=1024, keep=4, experts=32, top=4, ff=512,
+              shared=1024, vocab=32000),
+    "m": dict(width=2048, layers=8, m_heads=64, m_vdim=64, state=128, groups=8, a_heads=32, a_kv=8, dim=128, vdim=128, window=2048, keep=4, experts=64, top=6, ff=768,
+              shared=2048, vocab=32000),
+}
+
+
+def hybrid_leg(a, dev):
+    """`--hybrid SIZE`: prefill and decode throughput of a layer-list decoder (mistralrs_amd.hybrid: state-space + windowed-attention mixers, routed experts; bf16 weights,
+    random) beside the closest model the package had before -- the Llama runner with Mixtral-style sparse layers -- at equal width, depth, expert count / size and
+    vocabulary (Q4_K_M blocks: that runner serves quantized weights only).  Fractions: decode = bytes a step must read (active weights + states + pages) / 8 TB/s over
+    the measured step; prefill = 2 x active parameters x tokens (+ attention) / 2.5 PFLOP/s over the measured pass."""
+    import torch
+    from mistralrs_amd.hybrid import (AttentionSpec, HybridCache, HybridDecoder, HybridSpec, LayerSpec, Mamba2Spec, MoeSpec, RaggedBatch, RotarySpec, synthetic_weights)
+    z = HYBRID_SIZES[a.hybrid]
+    W = z["width"]
+    layers = []
+    for i in range(z["layers"]):
+        ff = MoeSpec(z["experts"], z["top"], z["ff"], z["shared"])
+        if i % 4 == 3:
+            mx = AttentionSpec(z["a_heads"], z["a_kv"], z["dim"], z["vdim"], z["dim"] ** -0.5, z["window"], z["keep"], RotarySpec(z["dim"] // 2, 500000.0, None))
+            layers.append(LayerSpec("attention", mx, ff, f"l{i}."))
+        else:
+            layers.append(LayerSpec("mamba2", Mamba2Spec(z["m_heads"], z["m_vdim"], z["state"], z["groups"], 4, z["groups"]), ff, f"l{i}."))
+    spec = HybridSpec(z["vocab"], W, 1e-6, layers)
+    prompts = [512, 2048]
+    batches = [1, 8]
+    bs = 32
+    max_tok = max(prompts) + a.warmup + a.steps + 64
+    model = HybridDecoder(spec, dev, "bfloat16", num_blocks=max(batches) * (-(-max_tok // bs) + 1) + 2, block_size=bs, state_slots=max(batches))
+    model.load_weights(synthetic_weights(spec, dev, 0))
+    cache = HybridCache(model)
+    e = 2
+
+    def active_weight_bytes(rows):
+        tot = e * z["vocab"] * W  # head (the embedding is one row per token)
+        for ls in spec.layers:
+            m = ls.mixer
+            if isinstance(m, Mamba2Spec):
+                tot += e * W * (2 * m.inner + 2 * m.groups * m.state + m.heads) + e * W * m.inner
+            else:
+                tot += e * W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + e * W * m.heads * m.vdim
+            f = ls.ff
+            tot += e * 3 * W * f.ff * min(f.experts, rows * f.top) + e * 3 * W * f.shared_ff + 4 * W * (f.experts + 1)
+        return tot
+
+    def flops_per_token(ctx):
+        tot = 2 * z["vocab"] * W
+        for ls in spec.layers:
+            m = ls.mixer
+            if isinstance(m, Mamba2Spec):
+                tot += 2 * W * (2 * m.inner + 2 * m.groups * m.state + m.heads) + 2 * W * m.inner + 6 * m.inner * m.state
+            else:
+                tot += 2 * W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + 2 * W * m.heads * m.vdim + 2 * m.heads * (m.dim + m.vdim) * min(ctx, m.window + m.keep_first)
+            tot += 2 * 3 * W * (ls.ff.ff * ls.ff.top + ls.ff.shared_ff)
+        return tot
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    out = {"model": f"hybrid-{a.hybrid}", "sizes": z, "dtype": "bf16", "weights": "random, drawn on the device", "prefill": {}, "decode": {}}
+    with torch.no_grad():
+        for T in prompts:
+            assert cache.reserve(1, T)
+            b = RaggedBatch.build([cache.entry(1, [(1000 + i) % z["vocab"] for i in range(T)], 0, [T - 1])], bs, dev)
+            t = timed(lambda: model.forward_batch(b), 3)
+            out["prefill"][str(T)] = {"tokens_per_sec": round(T / t, 1), "ms": round(1e3 * t, 3), "mfma_frac": round(T * flops_per_token(T / 2) / t / MFMA_PEAK, 4)}
+            cache.release(1)
+        ctx = 512
+        for nb in batches:
+            for r in range(nb):
+                assert cache.reserve(r + 1, ctx + a.warmup + a.steps + 2)
+            pre = RaggedBatch.build([cache.entry(r + 1, [(1000 + i + r) % z["vocab"] for i in range(ctx)], 0, []) for r in range(nb)], bs, dev)
+            model.forward_batch(pre)
+            g = model.capture_decode(nb, -(-(ctx + a.warmup + a.steps + 2) // bs))
+            pos = ctx
+
+            def step():
+                nonlocal pos
+                g.replay([cache.entry(r + 1, [7 + r], pos) for r in range(nb)])
+                pos += 1
+            for _ in range(a.warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(a.steps):
+                step()
+            torch.cuda.synchronize()
+            t = (time.perf_counter() - t0) / a.steps
+            kv = sum(e * min(pos, l.mixer.window + l.mixer.keep_first) * l.mixer.kv_heads * (l.mixer.dim + l.mixer.vdim) for l in spec.layers if isinstance(l.mixer, AttentionSpec))
+            nbytes = active_weight_bytes(nb) + nb * (2 * model.state_bytes_per_slot() + kv)
+            out["decode"][f"batch{nb}"] = {"tokens_per_sec": round(nb / t, 1), "ms_per_step": round(1e3 * t, 4), "step_bytes": int(nbytes),
+                                           "hbm_frac": round(nbytes / t / HBM_PEAK, 4)}
+            for r in range(nb):
+                cache.release(r + 1)
+    del model, cache
+    torch.cuda.empty_cache()
+    # ---- the closest earlier model at equal size
+    try:
+        if a.hybrid_no_llama:
+            raise RuntimeError("skipped (--hybrid-no-llama)")
+        from mistralrs_amd.llama import LlamaConfig
+        heads = W // 128
+        for T in prompts[:1] if a.hybrid_quick else prompts:
+            max_ctx = (T + a.warmup + a.steps + 2 + 63) // 64 * 64
+            cfg = LlamaConfig(hidden_size=W, intermediate_size=z["ff"], num_layers=z["layers"], num_heads=heads, num_kv_heads=max(1, heads // 4), vocab_size=z["vocab"],
+                              max_batch=1, max_context_len=max_ctx, max_position_embeddings=max(8192, max_ctx), num_experts=z["experts"], num_experts_per_tok=z["top"])
+            lm = build_model(cfg, dev, seed=0, max_new_tokens=a.warmup + a.steps + 8, weights="blocks")
+            r = timed_run(lm, cfg, T, a.steps, a.warmup, 1, torch.cuda.synchronize, 1, dev)
+            sb = lm.decode_bytes(1, int(T + a.warmup + a.steps / 2))
+            out.setdefault("llama_moe_q4_k_m_equal_size", {})[str(T)] = {
+                "prefill_tokens_per_sec": round(T / r["ttft"], 1), "prefill_mfma_frac": round(r["prefill_flops"] / r["ttft"] / MFMA_PEAK, 4),
+                "decode_tokens_per_sec": round(a.steps / r["t_all"], 1), "decode_hbm_frac": round(sb * (a.steps / r["t_all"]) / HBM_PEAK, 4),
+                "prefill_arithmetic": "decode engine's (exact)" if lm.prefill_is_exact else "bf16-operand MFMA", "decode_path": lm.decode_path}
+            del lm
+            torch.cuda.empty_cache()
+    except Exception as ex:  # a reported side leg
+        out["llama_moe_q4_k_m_equal_size"] = {"failed": f"{type(ex).__name__}: {str(ex)[:300]}"}
+    d1 = out["decode"]["batch1"]
+    print(json.dumps({"metric": "hybrid_decode_tokens_per_sec", "value": d1["tokens_per_sec"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": d1["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"model": out["model"], "global_batch": 1, "seq_len": 512, "parallelism": "tp1"}, "hybrid": out}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -596,7 +728,18 @@ def main():
     ap.add_argument("--parity-positions", type=int, default=16, help="greedy positions of the CPU-path parity leg")
     ap.add_argument("--quant", choices=["q4_k_m", "q8_0_isq"], default="q4_k_m",
                     help="q8_0_isq = BASELINE configs[2]: every linear quantized in situ from bf16 weights to Q8_0 on the GPU (mistralrs_amd.isq, role of generate_isq!)")
+    ap.add_argument("--hybrid", choices=sorted(HYBRID_SIZES), default=None,
+                    help="instead of the default workload: a layer-list decoder (state-space + windowed-attention mixers, routed experts; bf16) of the given size beside the Llama runner at equal size")
+    ap.add_argument("--hybrid-no-llama", action="store_true", help="--hybrid: skip the equal-size Llama leg (profiling runs)")
+    ap.add_argument("--hybrid-quick", action="store_true", help="--hybrid: the equal-size Llama leg at the short prompt only")
     a = ap.parse_args()
+    if a.hybrid:
+        import torch
+        dev = torch.device("cuda", 0)
+        torch.cuda.set_device(dev)
+        if a.steps == 256:
+            a.steps = 128
+        return hybrid_leg(a, dev)
 
     if a.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # driver contract: `python bench.py --gpus N` must use N GPUs -- re-launch ourselves as one process per GPU (mistralrs-core/src/distributed.rs:569-795

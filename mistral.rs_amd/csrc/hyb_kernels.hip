@@ -42,19 +42,26 @@ template <class T> __global__ void __launch_bounds__(256) embed_kernel(const int
 }
 
 // ---------------------------------------------------------------------------------- x / sqrt(mean(x^2) + eps) * (w | 1 + w); grid.y = equal parts of the row
+// gate (optional, [rows, ldg]): the row is multiplied by silu(gate) BEFORE its root mean square is taken
 template <class T> __global__ void __launch_bounds__(256) rmsnorm_kernel(const float *__restrict__ x, int ldx, const float *__restrict__ w, T *__restrict__ out, float *__restrict__ out32,
-                                                                          float *__restrict__ rstd, int part, float eps, int one_plus, int ldo) {
+                                                                          float *__restrict__ rstd, int part, float eps, int one_plus, int ldo, const float *__restrict__ gate, int ldg) {
   __shared__ float red[4];
+  extern __shared__ float row[];  // the (gated) part, when a gate is given: silu is evaluated once
   const int t = blockIdx.x, g = blockIdx.y;
   const float *xr = x + (size_t)t * ldx + (size_t)g * part;
+  const float *gr = gate ? gate + (size_t)t * ldg + (size_t)g * part : nullptr;
   float s = 0.f;
-  for (int c = threadIdx.x; c < part; c += 256) s = fmaf(xr[c], xr[c], s);
+  for (int c = threadIdx.x; c < part; c += 256) {
+    float v = xr[c];
+    if (gr) { v *= silu_f(gr[c]); row[c] = v; }
+    s = fmaf(v, v, s);
+  }
   s = block_sum_256(s, red);
   const float inv = 1.0f / sqrtf(s / (float)part + eps);
   if (rstd && threadIdx.x == 0) rstd[(size_t)t * gridDim.y + g] = inv;
   for (int c = threadIdx.x; c < part; c += 256) {
     const float wv = w[(size_t)g * part + c];
-    const float v = xr[c] * inv * (one_plus ? 1.0f + wv : wv);
+    const float v = (gr ? row[c] : xr[c]) * inv * (one_plus ? 1.0f + wv : wv);
     if (out) out[(size_t)t * ldo + (size_t)g * part + c] = from_f<T>(v);
     if (out32) out32[(size_t)t * ldo + (size_t)g * part + c] = v;
   }
@@ -105,19 +112,29 @@ __global__ void __launch_bounds__(256) conv_state_kernel(const float *__restrict
 }
 
 // ---------------------------------------------------------------------------------- state-space-duality recurrence, token by token, f32 state carried in a slot
-//   dt = softplus(dt_raw + dt_bias_h);  S <- exp(-exp(A_log_h) dt) S + dt B x^T  (S: N x P);  y = S^T C + D_h x;  out = y * silu(z)
-// One wave per (entry, head, tile of P): lane = (p, r), r in [0, R) owns the state rows n = r + R k; the sum over n closes with R-lane butterflies.  No LDS, no barrier: the
-// per-token chain is the FMA pass plus log2(R) shuffles, and the next token's operands are requested before the current one is used.
+//   dt = softplus(dt_raw + dt_bias_h);  S <- exp(-exp(A_log_h) dt) S + dt B x^T  (S: N x P);  y = S^T C + D_h x          (the gate and the norm follow in rmsnorm_kernel)
+// Step sizes and decays of all rows first (ssd_steps_kernel: the transcendental functions leave the serial chain).  Then one wave per (entry, head, tile of P):
+// lane = (p, r), r in [0, R) owns the state rows n in [r K, r K + K); the sum over n closes with R-lane butterflies.  No LDS, no barrier: the per-token chain is the FMA
+// pass plus log2(R) shuffles, and the next token's operands are requested before the current one is used.
 struct ScanArgs {
   const float *xbc;   // [rows, C]: x [heads * P] | B [G * N] | C [G * N] after convolution + SiLU
-  const float *u;     // [rows, ldu] projection: z at column 0, dt_raw at column dt_col
+  const float *u;     // [rows, ldu] projection: dt_raw at column dt_col
   const float *dt_bias, *A_log, *D;
+  float *steps;       // [rows, heads, 2]: dt, decay
   float *state;       // [slots, heads, N, P]
   float *out;         // [rows, heads * P]
   const int *seq_start, *seq_pos0, *seq_slot;
-  int C, ldu, dt_col, heads, P, N, G;
+  int C, ldu, dt_col, heads, P, N, G, rows;
 };
-template <int R, int MAXK> __global__ void __launch_bounds__(64) ssd_scan_kernel(ScanArgs a) {
+__global__ void __launch_bounds__(256) ssd_steps_kernel(ScanArgs a) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.rows * a.heads) return;
+  const int t = i / a.heads, h = i % a.heads;
+  const float dt = softplus_f(a.u[(size_t)t * a.ldu + a.dt_col + h] + a.dt_bias[h]);
+  a.steps[2 * (size_t)i] = dt;
+  a.steps[2 * (size_t)i + 1] = expf(-expf(a.A_log[h]) * dt);
+}
+template <int R, int K, bool VEC> __global__ void __launch_bounds__(64) ssd_scan_kernel(ScanArgs a) {
   constexpr int PT = 64 / R;
   const int lane = threadIdx.x, r = lane % R, p = blockIdx.x * PT + lane / R;
   const int h = blockIdx.y, s = blockIdx.z;
@@ -126,48 +143,57 @@ template <int R, int MAXK> __global__ void __launch_bounds__(64) ssd_scan_kernel
   const bool live = p < a.P;
   const int pc = live ? p : a.P - 1;
   const int g = h / (a.heads / a.G), inner = a.heads * a.P;
-  const int nk = (a.N - r + R - 1) / R;  // rows n = r + R k < N
+  int nk = a.N - r * K;  // this lane's rows n = r K + k, k < nk
+  nk = nk < 0 ? 0 : (nk > K ? K : nk);
   float *st = a.state + (((size_t)a.seq_slot[s] * a.heads + h) * a.N) * a.P;
-  float S[MAXK];
+  float S[K];
 #pragma unroll
-  for (int k = 0; k < MAXK; ++k) S[k] = (k < nk && a.seq_pos0[s] > 0) ? st[(size_t)(r + R * k) * a.P + pc] : 0.f;
-  const float Ah = -expf(a.A_log[h]), Dh = a.D[h], bias = a.dt_bias[h];
-  const int bcol = inner + g * a.N, ccol = inner + a.G * a.N + g * a.N;
-  float Bc[MAXK], Cc[MAXK], Bn[MAXK], Cn[MAXK], xv, dtr, zv, xv_n = 0.f, dtr_n = 0.f, zv_n = 0.f;
-  auto request = [&](int row, float *B_, float *C_, float &x_, float &d_, float &z_) {
+  for (int k = 0; k < K; ++k) S[k] = (k < nk && a.seq_pos0[s] > 0) ? st[(size_t)(r * K + k) * a.P + pc] : 0.f;
+  const float Dh = a.D[h];
+  const int bcol = inner + g * a.N + r * K, ccol = inner + a.G * a.N + g * a.N + r * K;
+  float Bc[K], Cc[K], Bn[K], Cn[K], xv, dt, dec, xv_n = 0.f, dt_n = 0.f, dec_n = 0.f;
+  auto request = [&](int row, float *B_, float *C_, float &x_, float &d_, float &e_) {
     const float *xr = a.xbc + (size_t)row * a.C;
+    if (VEC) {
 #pragma unroll
-    for (int k = 0; k < MAXK; ++k) {
-      const int n = r + R * k;
-      B_[k] = k < nk ? xr[bcol + n] : 0.f;
-      C_[k] = k < nk ? xr[ccol + n] : 0.f;
+      for (int k = 0; k < K; k += 4) {
+        float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f), c4 = b4;
+        if (k < nk) { b4 = *(const float4 *)(xr + bcol + k); c4 = *(const float4 *)(xr + ccol + k); }
+        B_[k] = b4.x; B_[k + 1] = b4.y; B_[k + 2] = b4.z; B_[k + 3] = b4.w;
+        C_[k] = c4.x; C_[k + 1] = c4.y; C_[k + 2] = c4.z; C_[k + 3] = c4.w;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        B_[k] = k < nk ? xr[bcol + k] : 0.f;
+        C_[k] = k < nk ? xr[ccol + k] : 0.f;
+      }
     }
     x_ = xr[h * a.P + pc];
-    d_ = a.u[(size_t)row * a.ldu + a.dt_col + h];
-    z_ = a.u[(size_t)row * a.ldu + h * a.P + pc];
+    const float2 de = *(const float2 *)(a.steps + 2 * ((size_t)row * a.heads + h));
+    d_ = de.x; e_ = de.y;
   };
-  request(r0, Bc, Cc, xv, dtr, zv);
+  request(r0, Bc, Cc, xv, dt, dec);
   for (int i = 0; i < len; ++i) {
-    if (i + 1 < len) request(r0 + i + 1, Bn, Cn, xv_n, dtr_n, zv_n);
-    const float dt = softplus_f(dtr + bias);
-    const float decay = expf(Ah * dt), dx = dt * xv;
+    if (i + 1 < len) request(r0 + i + 1, Bn, Cn, xv_n, dt_n, dec_n);
+    const float dx = dt * xv;
     float part = 0.f;
 #pragma unroll
-    for (int k = 0; k < MAXK; ++k) {
-      S[k] = fmaf(decay, S[k], dx * Bc[k]);
+    for (int k = 0; k < K; ++k) {
+      S[k] = fmaf(dec, S[k], dx * Bc[k]);
       part = fmaf(S[k], Cc[k], part);
     }
 #pragma unroll
     for (int m = 1; m < R; m <<= 1) part += __shfl_xor(part, m, 64);
-    if (r == 0 && live) a.out[(size_t)(r0 + i) * inner + h * a.P + p] = fmaf(Dh, xv, part) * silu_f(zv);
+    if (r == 0 && live) a.out[(size_t)(r0 + i) * inner + h * a.P + p] = fmaf(Dh, xv, part);
 #pragma unroll
-    for (int k = 0; k < MAXK; ++k) { Bc[k] = Bn[k]; Cc[k] = Cn[k]; }
-    xv = xv_n; dtr = dtr_n; zv = zv_n;
+    for (int k = 0; k < K; ++k) { Bc[k] = Bn[k]; Cc[k] = Cn[k]; }
+    xv = xv_n; dt = dt_n; dec = dec_n;
   }
   if (live)
 #pragma unroll
-    for (int k = 0; k < MAXK; ++k)
-      if (k < nk) st[(size_t)(r + R * k) * a.P + p] = S[k];
+    for (int k = 0; k < K; ++k)
+      if (k < nk) st[(size_t)(r * K + k) * a.P + p] = S[k];
 }
 
 // ---------------------------------------------------------------------------------- query / key norm over the whole projection, partial interleaved rotary, K / V page write
@@ -303,45 +329,81 @@ template <class T, int DVC> __global__ void __launch_bounds__(64) paged_window_a
 }
 
 // ---------------------------------------------------------------------------------- mixture of experts: routing, dispatch, gather, GLU, combine
-// z [rows, ldz]: E router logits (+ the shared expert's gate logit at column E when has_gate).  score = sigmoid(z); the `top` largest (ties: the lower index), weights = scores.
-__global__ void __launch_bounds__(256) route_sigmoid_topk_kernel(const float *__restrict__ z, int ldz, int rows, int E, int top, int has_gate, int *__restrict__ ids,
+// Router: one workgroup per row.  logits z_e = w_e . h in f32 (a wave per expert, lanes over the width, butterfly sum), score = sigmoid(z); the `top` largest (ties: the
+// lower index), weights = the scores, un-renormalised; row E of the weight (when has_gate) is the shared expert's gate: gate[t] = sigmoid(w_E . h).
+__global__ void __launch_bounds__(256) route_sigmoid_topk_kernel(const float *__restrict__ h, const float *__restrict__ wr, int W, int E, int top, int has_gate, int *__restrict__ ids,
                                                                  float *__restrict__ wts, float *__restrict__ gate) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= rows) return;
-  const float *zr = z + (size_t)t * ldz;
+  extern __shared__ float z[];  // [E + 1]
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float *hr = h + (size_t)t * W;
+  for (int e = wave; e < E + (has_gate ? 1 : 0); e += 4) {
+    const float *w = wr + (size_t)e * W;
+    float acc = 0.f;
+    for (int k = lane; k < W; k += 64) acc = fmaf(hr[k], w[k], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) z[e] = acc;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  if (has_gate && lane == 0) gate[t] = sigmoid_f(z[E]);
   for (int k = 0; k < top; ++k) {
-    int best = -1;
     float bv = -FLT_MAX;
-    for (int e = 0; e < E; ++e) {
-      bool taken = false;
-      for (int j = 0; j < k; ++j) taken |= ids[(size_t)t * top + j] == e;
-      if (!taken && (best < 0 || zr[e] > bv)) { best = e; bv = zr[e]; }
+    int be = 0x7fffffff;
+    for (int e = lane; e < E; e += 64)
+      if (z[e] > bv) { bv = z[e]; be = e; }  // ascending e: the first of equals stays
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) {
+      const float ov = __shfl_xor(bv, m, 64);
+      const int oe = __shfl_xor(be, m, 64);
+      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
     }
-    ids[(size_t)t * top + k] = best;
-    wts[(size_t)t * top + k] = sigmoid_f(bv);
+    if (lane == 0) {
+      ids[(size_t)t * top + k] = be;
+      wts[(size_t)t * top + k] = sigmoid_f(bv);
+    }
+    if ((be & 63) == lane) z[be] = -FLT_MAX;  // taken: written by the lane that reads this entry in the next round (every lane holds the same `be` after the butterfly)
   }
-  if (has_gate) gate[t] = sigmoid_f(zr[E]);
 }
-// stable counting sort of the routes by expert: bounds [E + 1], sorted_route [R] (route index = token * top + k), route_pos [R] (its inverse), sorted_expert [R]
-__global__ void __launch_bounds__(1024) moe_dispatch_kernel(const int *__restrict__ ids, int R, int E, int *__restrict__ bounds, int *__restrict__ sorted_route,
-                                                           int *__restrict__ route_pos, int *__restrict__ sorted_expert) {
-  extern __shared__ int cnt[];  // [E + 1]
-  for (int e = threadIdx.x; e < E; e += 1024) {
-    int c = 0;
-    for (int r = 0; r < R; ++r) c += ids[r] == e;
-    cnt[e] = c;
+// stable counting sort of the routes by expert, one workgroup per expert: bounds [E + 1], sorted_route [R] (route index = token * top + k), route_pos [R] (its inverse),
+// sorted_expert [R].  Every workgroup counts the routes below its expert (its base) and its own, then places its routes in ascending route order.
+__global__ void __launch_bounds__(256) moe_dispatch_kernel(const int *__restrict__ ids, int R, int E, int *__restrict__ bounds, int *__restrict__ sorted_route,
+                                                          int *__restrict__ route_pos, int *__restrict__ sorted_expert) {
+  __shared__ int red[2][4];
+  __shared__ int wcnt[4];
+  const int e = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  int less = 0, eq = 0;
+  for (int r = tid; r < R; r += 256) {
+    const int id = ids[r];
+    less += id < e;
+    eq += id == e;
   }
+  less = wave_sum(less);
+  eq = wave_sum(eq);
+  if (lane == 0) { red[0][wave] = less; red[1][wave] = eq; }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int e = 0; e < E; ++e) { const int c = cnt[e]; cnt[e] = run; bounds[e] = run; run += c; }
-    bounds[E] = run;
+  const int base = red[0][0] + red[0][1] + red[0][2] + red[0][3], cnt = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+  if (tid == 0) {
+    bounds[e] = base;
+    if (e == E - 1) bounds[E] = base + cnt;
   }
-  __syncthreads();
-  for (int e = threadIdx.x; e < E; e += 1024) {
-    int at = cnt[e];
-    for (int r = 0; r < R; ++r)
-      if (ids[r] == e) { sorted_route[at] = r; route_pos[r] = at; sorted_expert[at] = e; ++at; }
+  if (cnt == 0) return;
+  int running = base;
+  for (int r0 = 0; r0 < R; r0 += 256) {
+    const int r = r0 + tid;
+    const bool mine = r < R && ids[r] == e;
+    const unsigned long long bal = __ballot(mine);
+    if (lane == 0) wcnt[wave] = __popcll(bal);
+    __syncthreads();
+    int off = running;
+    for (int w = 0; w < wave; ++w) off += wcnt[w];
+    if (mine) {
+      const int at = off + __popcll(bal & ((1ull << lane) - 1ull));
+      sorted_route[at] = r;
+      route_pos[r] = at;
+      sorted_expert[at] = e;
+    }
+    running += wcnt[0] + wcnt[1] + wcnt[2] + wcnt[3];
+    __syncthreads();
   }
 }
 // row i of the expert-sorted operand = weight of its route * the token's normed row (f32), rounded once to T
@@ -393,12 +455,14 @@ extern "C" int mrs_hyb_embed(const int *tokens, const void *table, float *x, int
 
 // parts > 1: every row is normed in `parts` equal pieces, each by its own root mean square.  out (dtype) and / or out32 (f32) receive the result, rstd [rows, parts] the 1 / rms.
 extern "C" int mrs_hyb_rmsnorm(const float *x, int ldx, const float *w, void *out, float *out32, float *rstd, int rows, int width, int parts, float eps, int one_plus, int dtype,
-                               void *stream) {
+                               const float *gate, int ldg, void *stream) {
   if (rows <= 0) return 0;
   if (parts <= 0 || width % parts) return fail("mrs_hyb_rmsnorm: the row does not split into equal parts");
   dim3 grid(rows, parts);
-  if (dtype == 1) hipLaunchKernelGGL(rmsnorm_kernel<mrs::bf16_t>, grid, dim3(256), 0, S_(stream), x, ldx, w, (mrs::bf16_t *)out, out32, rstd, width / parts, eps, one_plus, width);
-  else if (dtype == 2) hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, dim3(256), 0, S_(stream), x, ldx, w, (float *)out, out32, rstd, width / parts, eps, one_plus, width);
+  const size_t lds = gate ? (size_t)(width / parts) * 4 : 0;
+  if (lds > 60000) return fail("mrs_hyb_rmsnorm: a gated part above 15000 values");
+  if (dtype == 1) hipLaunchKernelGGL(rmsnorm_kernel<mrs::bf16_t>, grid, dim3(256), lds, S_(stream), x, ldx, w, (mrs::bf16_t *)out, out32, rstd, width / parts, eps, one_plus, width, gate, ldg);
+  else if (dtype == 2) hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, dim3(256), lds, S_(stream), x, ldx, w, (float *)out, out32, rstd, width / parts, eps, one_plus, width, gate, ldg);
   else return fail("mrs_hyb_rmsnorm: dtype");
   return ok_or("mrs_hyb_rmsnorm");
 }
@@ -413,12 +477,17 @@ extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const
   return ok_or("mrs_hyb_conv_silu");
 }
 
+/* steps: scratch [rows, heads, 2] f32 */
 extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, float *state, float *out, const int *seq_start,
-                                const int *seq_pos0, const int *seq_slot, int entries, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream) {
-  if (entries <= 0) return 0;
+                                const int *seq_pos0, const int *seq_slot, float *steps, int rows, int entries, int C, int ldu, int dt_col, int heads, int P, int N, int G,
+                                void *stream) {
+  if (entries <= 0 || rows <= 0) return 0;
   if (heads <= 0 || G <= 0 || heads % G || P <= 0 || N <= 0) return fail("mrs_hyb_ssd_scan: bad head / group sizes");
-  ScanArgs a{xbc, u, dt_bias, A_log, D, state, out, seq_start, seq_pos0, seq_slot, C, ldu, dt_col, heads, P, N, G};
-#define MRS_SCAN(R, K) hipLaunchKernelGGL((ssd_scan_kernel<R, K>), dim3((P + 64 / R - 1) / (64 / R), heads, entries), dim3(64), 0, S_(stream), a)
+  ScanArgs a{xbc, u, dt_bias, A_log, D, steps, state, out, seq_start, seq_pos0, seq_slot, C, ldu, dt_col, heads, P, N, G, rows};
+  hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
+  const bool vec = C % 4 == 0 && (heads * P) % 4 == 0 && N % 4 == 0 && ((uintptr_t)xbc % 16) == 0;
+#define MRS_SCAN(R, K) do { if (vec) hipLaunchKernelGGL((ssd_scan_kernel<R, K, true>), dim3((P + 64 / R - 1) / (64 / R), heads, entries), dim3(64), 0, S_(stream), a); \
+                            else hipLaunchKernelGGL((ssd_scan_kernel<R, K, false>), dim3((P + 64 / R - 1) / (64 / R), heads, entries), dim3(64), 0, S_(stream), a); } while (0)
   if (N <= 16) MRS_SCAN(2, 8);
   else if (N <= 64) MRS_SCAN(4, 16);
   else if (N <= 128) MRS_SCAN(4, 32);
@@ -457,16 +526,18 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
   return ok_or("mrs_hyb_paged_window_attn");
 }
 
-extern "C" int mrs_hyb_route_sigmoid_topk(const float *z, int ldz, int rows, int E, int top, int has_gate, int *ids, float *wts, float *gate, void *stream) {
+/* h [rows, W] f32 (contiguous), wr [E (+ 1), W] f32 */
+extern "C" int mrs_hyb_route_sigmoid_topk(const float *h, const float *wr, int rows, int W, int E, int top, int has_gate, int *ids, float *wts, float *gate, void *stream) {
   if (rows <= 0) return 0;
-  if (top < 1 || top > E) return fail("mrs_hyb_route_sigmoid_topk: 1 <= top <= experts");
-  hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3((rows + 255) / 256), dim3(256), 0, S_(stream), z, ldz, rows, E, top, has_gate, ids, wts, gate);
+  if (top < 1 || top > E || E > 8192) return fail("mrs_hyb_route_sigmoid_topk: 1 <= top <= experts <= 8192");
+  hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3(rows), dim3(256), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, has_gate, ids, wts, gate);
   return ok_or("mrs_hyb_route_sigmoid_topk");
 }
 
 extern "C" int mrs_hyb_moe_dispatch(const int *ids, int R, int E, int *bounds, int *sorted_route, int *route_pos, int *sorted_expert, void *stream) {
   if (E <= 0 || E > 8192) return fail("mrs_hyb_moe_dispatch: 1 .. 8192 experts");
-  hipLaunchKernelGGL(moe_dispatch_kernel, dim3(1), dim3(1024), (size_t)(E + 1) * 4, S_(stream), ids, R, E, bounds, sorted_route, route_pos, sorted_expert);
+  if (R <= 0) return 0;
+  hipLaunchKernelGGL(moe_dispatch_kernel, dim3(E), dim3(256), 0, S_(stream), ids, R, E, bounds, sorted_route, route_pos, sorted_expert);
   return ok_or("mrs_hyb_moe_dispatch");
 }
 

@@ -30,12 +30,12 @@ DTYPES = {"bfloat16": (1, torch.bfloat16), "float32": (2, torch.float32)}
 
 _SIGS = {
     "mrs_hyb_embed": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
-    "mrs_hyb_rmsnorm": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp],
+    "mrs_hyb_rmsnorm": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _i, _vp],
     "mrs_hyb_conv_silu": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
-    "mrs_hyb_ssd_scan": [_vp] * 10 + [_i] * 8 + [_vp],
+    "mrs_hyb_ssd_scan": [_vp] * 11 + [_i] * 10 + [_vp],
     "mrs_hyb_qk_norm_rope_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "mrs_hyb_paged_window_attn": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp],
-    "mrs_hyb_route_sigmoid_topk": [_vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp],
+    "mrs_hyb_route_sigmoid_topk": [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp],
     "mrs_hyb_moe_dispatch": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp],
     "mrs_hyb_moe_gather": [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp],
     "mrs_hyb_glu_silu": [_vp, _vp, _i, _i, _i, _vp],
@@ -267,9 +267,10 @@ class Mamba2Mixer(_Module):
         _call("mrs_hyb_conv_silu", u[:, s.inner:], u.stride(0), self.conv_w, self.conv_b, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, xbc,
               T, b.entries, s.conv_channels, s.conv)
         y = torch.empty(T, s.inner, dtype=torch.float32, device=m.device)
-        _call("mrs_hyb_ssd_scan", xbc, u, self.dt_bias, self.A_log, self.D, self.ssm_state, y, b.seq_start, b.seq_pos0, b.seq_slot, b.entries, s.conv_channels,
+        steps = torch.empty(T, s.heads, 2, dtype=torch.float32, device=m.device)
+        _call("mrs_hyb_ssd_scan", xbc, u, self.dt_bias, self.A_log, self.D, self.ssm_state, y, b.seq_start, b.seq_pos0, b.seq_slot, steps, T, b.entries, s.conv_channels,
               u.stride(0), s.inner + s.conv_channels, s.heads, s.vdim, s.state, s.groups)
-        yn = m.norm(y, self.norm, one_plus=False, parts=s.norm_groups)
+        yn = m.norm(y, self.norm, one_plus=False, parts=s.norm_groups, gate=u)   # y * silu(z) (z = the first `inner` columns of u), then the grouped norm
         m.linear(yn, self.w_o, out=x, accumulate=True)
 
     def state_bytes_per_slot(self) -> int:
@@ -338,11 +339,10 @@ class SigmoidMoe(_Module):
         s, m = self.s, self.m
         T, W, dev = b.rows, m.spec.width, m.device
         R = T * s.top
-        z = m.linear(h32, self.w_router, dtype_code=2)
         ids = torch.empty(R, dtype=torch.int32, device=dev)
         wts = torch.empty(R, dtype=torch.float32, device=dev)
         gate = torch.empty(T, dtype=torch.float32, device=dev) if s.shared_ff else None
-        _call("mrs_hyb_route_sigmoid_topk", z, z.stride(0), T, s.experts, s.top, int(bool(s.shared_ff)), ids, wts, gate)
+        _call("mrs_hyb_route_sigmoid_topk", h32, self.w_router, T, W, s.experts, s.top, int(bool(s.shared_ff)), ids, wts, gate)
         meta = torch.empty(s.experts + 1 + 3 * R, dtype=torch.int32, device=dev)
         bounds, sorted_route, route_pos, sorted_expert = meta[:s.experts + 1], meta[s.experts + 1:][:R], meta[s.experts + 1 + R:][:R], meta[s.experts + 1 + 2 * R:][:R]
         _call("mrs_hyb_moe_dispatch", ids, R, s.experts, bounds, sorted_route, route_pos, sorted_expert)
@@ -427,11 +427,12 @@ class HybridDecoder:
         return model
 
     # ---- building blocks on the current stream
-    def norm(self, x, w, one_plus: bool, parts: int = 1, want32: bool = False):
+    def norm(self, x, w, one_plus: bool, parts: int = 1, want32: bool = False, gate=None):
+        """RMS norm of every row (in `parts` equal pieces); gate [rows, >= width]: the row is multiplied by silu(gate) first."""
         rows, width = x.shape
         out = torch.empty(rows, width, dtype=self.torch_dtype, device=self.device)
         out32 = torch.empty(rows, width, dtype=torch.float32, device=self.device) if want32 else None
-        _call("mrs_hyb_rmsnorm", x, x.stride(0), w, out, out32, None, rows, width, parts, self.spec.eps, int(one_plus), self.dt)
+        _call("mrs_hyb_rmsnorm", x, x.stride(0), w, out, out32, None, rows, width, parts, self.spec.eps, int(one_plus), self.dt, gate, gate.stride(0) if gate is not None else 0)
         return (out, out32) if want32 else out
 
     def linear(self, a, w, out=None, accumulate: bool = False, dtype_code: Optional[int] = None):
@@ -481,6 +482,11 @@ class HybridDecoder:
         _call("mrs_hyb_gather_rows", x, b.want, xs, n, sp.width)
         return self.linear(self.norm(xs, self.final_norm, one_plus=True), self.head)
 
+    # ---- decode steps as a HIP graph
+    def capture_decode(self, entries: int, max_blocks: int) -> "DecodeGraph":
+        """One decode step for `entries` sequences (one row each), captured into a HIP graph over static batch buffers: replays cost one launch instead of one per kernel."""
+        return DecodeGraph(self, entries, max_blocks)
+
     # ---- sizes
     def kv_bytes_per_token(self) -> int:
         e = 2 if self.dtype == "bfloat16" else 4
@@ -488,6 +494,110 @@ class HybridDecoder:
 
     def state_bytes_per_slot(self) -> int:
         return sum(l.mixer.state_bytes_per_slot() for l in self.layers if isinstance(l.mixer, Mamba2Mixer))
+
+
+class DecodeGraph:
+    """A captured decode step (role of pipeline/cuda_graph.rs in the reference): the batch description lives in static device buffers that `replay` refreshes with two
+    small host -> device copies; every kernel argument besides those buffers (row counts, table width) is fixed at capture.  Logits of all rows come back as a view of a
+    static buffer: consume them before the next replay."""
+
+    def __init__(self, model: HybridDecoder, entries: int, max_blocks: int):
+        self.m, self.n, self.mb = model, int(entries), int(max_blocks)
+        dev, n, mb = model.device, self.n, self.mb
+        self._ints = torch.zeros(3 * n + (n + 1) + 2 * n + n * mb, dtype=torch.int32, device=dev)
+        self._slots = torch.zeros(n, dtype=torch.int64, device=dev)
+        v, o = [], 0
+        for k in (n, n, n, n + 1, n, n, n * mb):
+            v.append(self._ints[o:o + k])
+            o += k
+        self.batch = RaggedBatch(n, n, mb, v[0], v[1], v[2], v[3], v[4], v[5], v[6].view(n, mb), self._slots, torch.arange(n, dtype=torch.int32, device=dev))
+        self._host = np.zeros(self._ints.numel(), dtype=np.int32)
+        self._host[3 * n:3 * n + n + 1] = np.arange(n + 1)          # seq_start: one row per entry
+        self._host[2 * n:3 * n] = 1                                  # positions >= 1 during warm-up: the slots' states are read, nothing is reset
+        self._host[n:2 * n] = np.arange(n)                           # tok_seq
+        self._ints.copy_(torch.from_numpy(self._host))
+        # warm-up outside capture (lazy module loads).  It really runs -- on state slot 0 and page slot 0, which may belong to a live sequence: put both back afterwards
+        keep = []
+        for l in model.layers:
+            mx = l.mixer
+            keep += [(t, t[0].clone()) for t in ((mx.conv_state, mx.ssm_state) if isinstance(mx, Mamba2Mixer) else (mx.k_cache, mx.v_cache))]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model.forward_batch(self.batch)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for t, saved in keep:
+            t[0].copy_(saved)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = model.forward_batch(self.batch)
+
+    def replay(self, entries: Sequence[dict]) -> torch.Tensor:
+        """entries as for RaggedBatch.build, one token each (`pos0` = the token's position)."""
+        n, mb, h = self.n, self.mb, self._host
+        if len(entries) != n:
+            raise ValueError(f"DecodeGraph: captured for {n} sequences, got {len(entries)}")
+        slots = np.zeros(n, dtype=np.int64)
+        bt = h[3 * n + (n + 1) + 2 * n:].reshape(n, mb)
+        bs = self.m.block_size
+        for s, e in enumerate(entries):
+            p, blocks = int(e["pos0"]), e["blocks"]
+            if len(e["tokens"]) != 1 or len(blocks) > mb or p // bs >= len(blocks):
+                raise ValueError("DecodeGraph: one token per entry, its page inside the captured table width")
+            h[s], h[2 * n + s] = e["tokens"][0], p
+            h[3 * n + (n + 1) + s], h[3 * n + (n + 1) + n + s] = p, int(e.get("slot") or 0)
+            bt[s, :len(blocks)] = blocks
+            slots[s] = blocks[p // bs] * bs + p % bs
+        self._ints.copy_(torch.from_numpy(h))
+        self._slots.copy_(torch.from_numpy(slots))
+        self.graph.replay()
+        return self.logits
+
+
+def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str], torch.Tensor]:
+    """`get(name)` for HybridDecoder.load_weights that draws every tensor on the device when it is asked for (benchmarks: there is no network for checkpoints).
+    Projections N(0, 1 / fan_in), norm weights around their neutral value, decays and step sizes in the range trained state-space models use."""
+    W = spec.width
+    g = torch.Generator(device=device).manual_seed(seed)
+    shapes: Dict[str, tuple] = {spec.embed: (spec.vocab, W), spec.head: (spec.vocab, W), spec.final_norm: (W,)}
+    for ls in spec.layers:
+        p, m = ls.prefix, ls.mixer
+        shapes[p + "norm1"] = (W,)
+        if isinstance(m, Mamba2Spec):
+            shapes.update({p + "mix.in": (2 * m.inner + 2 * m.groups * m.state + m.heads, W), p + "mix.conv": (m.conv_channels, m.conv), p + "mix.conv.b": (m.conv_channels,),
+                           p + "mix.dt_bias": (m.heads,), p + "mix.A_log": (m.heads,), p + "mix.D": (m.heads,), p + "mix.norm": (m.inner,), p + "mix.o": (W, m.inner)})
+        else:
+            shapes.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.kv_heads * m.dim, W), p + "mix.v": (m.kv_heads * m.vdim, W), p + "mix.q.norm": (m.heads * m.dim,),
+                           p + "mix.k.norm": (m.kv_heads * m.dim,), p + "mix.o": (W, m.heads * m.vdim)})
+        if ls.ff:
+            f = ls.ff
+            shapes[p + "norm2"], shapes[p + "mlp.router"] = (W,), (f.experts, W)
+            for e in range(f.experts):
+                shapes.update({f"{p}mlp.e{e}.gate": (f.ff, W), f"{p}mlp.e{e}.up": (f.ff, W), f"{p}mlp.e{e}.down": (W, f.ff)})
+            if f.shared_ff:
+                shapes.update({p + "mlp.shared.gate": (f.shared_ff, W), p + "mlp.shared.up": (f.shared_ff, W), p + "mlp.shared.down": (W, f.shared_ff), p + "mlp.shared.sg": (1, W)})
+
+    def get(name: str) -> torch.Tensor:
+        shape = shapes[name]
+        r = torch.randn(*shape, device=device, generator=g)
+        last = name.rsplit(".", 1)[-1]
+        if name.endswith(("q.norm", "k.norm")) or last == "D" or name.endswith("mix.norm"):
+            r = 1.0 + 0.1 * r
+        elif last in ("norm1", "norm2") or name == spec.final_norm:
+            r = 0.1 * r
+        elif last == "dt_bias":
+            r = -2.0 + 0.5 * r
+        elif last == "A_log":
+            r = 0.5 * r
+        elif last == "b":
+            r = 0.1 * r
+        elif last == "conv":
+            r = 0.4 * r
+        elif name != spec.embed:
+            r = r * (shape[-1] ** -0.5)
+        return r.to(torch.bfloat16)
+    return get
 
 
 SPEC_READERS: Dict[str, Callable[[dict], HybridSpec]] = {"Gekilix": gekilix_spec}
