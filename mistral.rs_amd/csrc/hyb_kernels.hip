@@ -111,11 +111,15 @@ __global__ void __launch_bounds__(256) conv_state_kernel(const float *__restrict
   }
 }
 
-// ---------------------------------------------------------------------------------- state-space-duality recurrence, token by token, f32 state carried in a slot
+// ---------------------------------------------------------------------------------- state-space-duality recurrence, f32 state carried in a slot
 //   dt = softplus(dt_raw + dt_bias_h);  S <- exp(-exp(A_log_h) dt) S + dt B x^T  (S: N x P);  y = S^T C + D_h x          (the gate and the norm follow in rmsnorm_kernel)
-// Step sizes and decays of all rows first (ssd_steps_kernel: the transcendental functions leave the serial chain).  Then one wave per (entry, head, tile of P):
-// lane = (p, r), r in [0, R) owns the state rows n in [r K, r K + K); the sum over n closes with R-lane butterflies.  No LDS, no barrier: the per-token chain is the FMA
-// pass plus log2(R) shuffles, and the next token's operands are requested before the current one is used.
+// Step sizes and decays of all rows first (ssd_steps_kernel: the transcendental functions leave the serial chain).  The rows of an entry are cut into segments (a table
+// the host builds); the recurrence is linear in S, so a long portion runs as
+//   A  every segment but an entry's last, from a ZERO state: its local end state L_k and the product d_k of its decays          (parallel over segments)
+//   B  init_(k+1) = d_k init_k + L_k, init_0 = the slot's state (zero for an entry that starts at position 0)                  (elementwise, serial over an entry's segments)
+//   C  every segment from its init state: the outputs; an entry's last segment leaves the slot's new state                     (parallel over segments)
+// and an entry of one segment (a decoded token, a short portion) is pass C alone.  Scan kernel: one wave per (segment, head, tile of P): lane = (p, r), r in [0, R) owns the
+// state rows n in [r K, r K + K); the sum over n closes with R-lane butterflies.  No LDS, no barrier; DEPTH tokens' operands are in flight in a ring of register stages.
 struct ScanArgs {
   const float *xbc;   // [rows, C]: x [heads * P] | B [G * N] | C [G * N] after convolution + SiLU
   const float *u;     // [rows, ldu] projection: dt_raw at column dt_col
@@ -123,7 +127,10 @@ struct ScanArgs {
   float *steps;       // [rows, heads, 2]: dt, decay
   float *state;       // [slots, heads, N, P]
   float *out;         // [rows, heads * P]
-  const int *seq_start, *seq_pos0, *seq_slot;
+  const int *seq_pos0, *seq_slot;
+  const int *seg_entry, *seg_row0, *seg_len, *ent_seg0;  // segment table: entry, first row, rows; first segment of every entry (+ the total)
+  float *carry;       // [segments, heads, N, P]: L_k, then init_(k+1)
+  float *decay;       // [segments, heads]: d_k
   int C, ldu, dt_col, heads, P, N, G, rows;
 };
 __global__ void __launch_bounds__(256) ssd_steps_kernel(ScanArgs a) {
@@ -134,63 +141,101 @@ __global__ void __launch_bounds__(256) ssd_steps_kernel(ScanArgs a) {
   a.steps[2 * (size_t)i] = dt;
   a.steps[2 * (size_t)i + 1] = expf(-expf(a.A_log[h]) * dt);
 }
-template <int R, int K, bool VEC> __global__ void __launch_bounds__(64) ssd_scan_kernel(ScanArgs a) {
+__global__ void __launch_bounds__(256) ssd_carry_kernel(ScanArgs a) {
+  const int e = blockIdx.x * 256 + threadIdx.x, h = blockIdx.y, s = blockIdx.z;
+  const int np = a.N * a.P;
+  if (e >= np) return;
+  const int z0 = a.ent_seg0[s], z1 = a.ent_seg0[s + 1];
+  if (z1 - z0 < 2) return;
+  float cur = a.seq_pos0[s] > 0 ? a.state[((size_t)a.seq_slot[s] * a.heads + h) * np + e] : 0.f;
+  for (int z = z0; z < z1 - 1; ++z) {
+    float *c = a.carry + ((size_t)z * a.heads + h) * np + e;
+    cur = fmaf(a.decay[(size_t)z * a.heads + h], cur, *c);
+    *c = cur;
+  }
+}
+struct ScanStage {
+  float x, dt, dec;
+};
+// LOCAL: pass A (zero start, no outputs, end state and decay product to `carry` / `decay`), else pass C
+template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launch_bounds__(64) ssd_scan_kernel(ScanArgs a) {
   constexpr int PT = 64 / R;
   const int lane = threadIdx.x, r = lane % R, p = blockIdx.x * PT + lane / R;
-  const int h = blockIdx.y, s = blockIdx.z;
-  const int r0 = a.seq_start[s], len = a.seq_start[s + 1] - r0;
-  if (len <= 0) return;
+  const int h = blockIdx.y, z = blockIdx.z;
+  const int s = a.seg_entry[z], r0 = a.seg_row0[z], len = a.seg_len[z];
+  const bool first = z == a.ent_seg0[s], last = z == a.ent_seg0[s + 1] - 1;
+  if (len <= 0 || (LOCAL && last)) return;
   const bool live = p < a.P;
   const int pc = live ? p : a.P - 1;
   const int g = h / (a.heads / a.G), inner = a.heads * a.P;
   int nk = a.N - r * K;  // this lane's rows n = r K + k, k < nk
   nk = nk < 0 ? 0 : (nk > K ? K : nk);
-  float *st = a.state + (((size_t)a.seq_slot[s] * a.heads + h) * a.N) * a.P;
+  const size_t np = (size_t)a.N * a.P;
+  float *st = a.state + ((size_t)a.seq_slot[s] * a.heads + h) * np;
+  const float *init = LOCAL ? nullptr : (first ? (a.seq_pos0[s] > 0 ? st : nullptr) : a.carry + ((size_t)(z - 1) * a.heads + h) * np);
   float S[K];
 #pragma unroll
-  for (int k = 0; k < K; ++k) S[k] = (k < nk && a.seq_pos0[s] > 0) ? st[(size_t)(r * K + k) * a.P + pc] : 0.f;
+  for (int k = 0; k < K; ++k) S[k] = (k < nk && init) ? init[(size_t)(r * K + k) * a.P + pc] : 0.f;
   const float Dh = a.D[h];
   const int bcol = inner + g * a.N + r * K, ccol = inner + a.G * a.N + g * a.N + r * K;
-  float Bc[K], Cc[K], Bn[K], Cn[K], xv, dt, dec, xv_n = 0.f, dt_n = 0.f, dec_n = 0.f;
-  auto request = [&](int row, float *B_, float *C_, float &x_, float &d_, float &e_) {
+  float B[DEPTH][K], Cv[DEPTH][K], prod = 1.0f;
+  ScanStage sg[DEPTH];
+  // unconditional requests (rows past the end re-read the last row; their step is made a no-op below): the waits before a stage's use then count exactly the
+  // requests issued after it
+  auto request = [&](int i, float *B_, float *C_, ScanStage &g_) {
+    const int row = r0 + (i < len ? i : len - 1);
     const float *xr = a.xbc + (size_t)row * a.C;
     if (VEC) {
 #pragma unroll
       for (int k = 0; k < K; k += 4) {
-        float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f), c4 = b4;
-        if (k < nk) { b4 = *(const float4 *)(xr + bcol + k); c4 = *(const float4 *)(xr + ccol + k); }
-        B_[k] = b4.x; B_[k + 1] = b4.y; B_[k + 2] = b4.z; B_[k + 3] = b4.w;
-        C_[k] = c4.x; C_[k + 1] = c4.y; C_[k + 2] = c4.z; C_[k + 3] = c4.w;
+        const int kk = k < nk ? k : 0;  // lanes past the state size re-read a valid group (nk is a multiple of 4 here)
+        const float4 b4 = *(const float4 *)(xr + (nk ? bcol : inner) + kk), c4 = *(const float4 *)(xr + (nk ? ccol : inner) + kk);
+        const bool on = k < nk;
+        B_[k] = on ? b4.x : 0.f; B_[k + 1] = on ? b4.y : 0.f; B_[k + 2] = on ? b4.z : 0.f; B_[k + 3] = on ? b4.w : 0.f;
+        C_[k] = on ? c4.x : 0.f; C_[k + 1] = on ? c4.y : 0.f; C_[k + 2] = on ? c4.z : 0.f; C_[k + 3] = on ? c4.w : 0.f;
       }
     } else {
 #pragma unroll
       for (int k = 0; k < K; ++k) {
-        B_[k] = k < nk ? xr[bcol + k] : 0.f;
-        C_[k] = k < nk ? xr[ccol + k] : 0.f;
+        const int kk = k < nk ? k : 0;
+        const float bv = xr[(nk ? bcol : inner) + kk], cv = xr[(nk ? ccol : inner) + kk];
+        B_[k] = k < nk ? bv : 0.f;
+        C_[k] = k < nk ? cv : 0.f;
       }
     }
-    x_ = xr[h * a.P + pc];
-    const float2 de = *(const float2 *)(a.steps + 2 * ((size_t)row * a.heads + h));
-    d_ = de.x; e_ = de.y;
+    g_.x = xr[h * a.P + pc];
+    const float *de = a.steps + 2 * ((size_t)row * a.heads + h);
+    const float d0 = de[0], d1 = de[1];
+    g_.dt = i < len ? d0 : 0.f;    // past the end: S <- 1 S + 0
+    g_.dec = i < len ? d1 : 1.f;
   };
-  request(r0, Bc, Cc, xv, dt, dec);
-  for (int i = 0; i < len; ++i) {
-    if (i + 1 < len) request(r0 + i + 1, Bn, Cn, xv_n, dt_n, dec_n);
-    const float dx = dt * xv;
-    float part = 0.f;
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-      S[k] = fmaf(dec, S[k], dx * Bc[k]);
-      part = fmaf(S[k], Cc[k], part);
+  for (int j = 0; j < DEPTH; ++j) request(j, B[j], Cv[j], sg[j]);
+  for (int i0 = 0; i0 < len; i0 += DEPTH) {
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) {
+      const int i = i0 + j;
+      const float dx = sg[j].dt * sg[j].x, dec = sg[j].dec, xv = sg[j].x;
+      float part = 0.f;
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        S[k] = fmaf(dec, S[k], dx * B[j][k]);
+        if (!LOCAL) part = fmaf(S[k], Cv[j][k], part);
+      }
+      if (LOCAL) prod *= dec;
+      if (DEPTH > 1 || i0 + DEPTH < len) request(i + DEPTH, B[j], Cv[j], sg[j]);
+      if (!LOCAL) {
+#pragma unroll
+        for (int m = 1; m < R; m <<= 1) part += __shfl_xor(part, m, 64);
+        if (r == 0 && live && i < len) a.out[(size_t)(r0 + i) * inner + h * a.P + p] = fmaf(Dh, xv, part);
+      }
     }
-#pragma unroll
-    for (int m = 1; m < R; m <<= 1) part += __shfl_xor(part, m, 64);
-    if (r == 0 && live) a.out[(size_t)(r0 + i) * inner + h * a.P + p] = fmaf(Dh, xv, part);
-#pragma unroll
-    for (int k = 0; k < K; ++k) { Bc[k] = Bn[k]; Cc[k] = Cn[k]; }
-    xv = xv_n; dt = dt_n; dec = dec_n;
   }
-  if (live)
+  if (LOCAL) {
+    if (blockIdx.x == 0 && lane == 0) a.decay[(size_t)z * a.heads + h] = prod;
+    st = a.carry + ((size_t)z * a.heads + h) * np;
+  }
+  if (live && (LOCAL || last))
 #pragma unroll
     for (int k = 0; k < K; ++k)
       if (k < nk) st[(size_t)(r * K + k) * a.P + p] = S[k];
@@ -270,10 +315,32 @@ struct AttnArgs {
   int H, G, D, Dv, block_size, max_blocks, window, keep_first;
   float scale;
 };
-template <class T, int DVC> __global__ void __launch_bounds__(64) paged_window_attn_kernel(AttnArgs a) {
-  extern __shared__ float lds[];  // q [D] | p [64] | key row index [64] as int
-  float *qs = lds, *ps = lds + a.D;
-  long long *rowbase = (long long *)(ps + 64 + ((a.D & 1) ? 1 : 0));
+template <class T> struct Ld;
+template <> struct Ld<bf16_t> {
+  static __device__ __forceinline__ void v8(const bf16_t *p, float *o) {
+    const int4 v = *(const int4 *)p;
+    const unsigned u[4] = {(unsigned)v.x, (unsigned)v.y, (unsigned)v.z, (unsigned)v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { o[2 * j] = __uint_as_float(u[j] << 16); o[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u); }
+  }
+  static __device__ __forceinline__ void v2(const bf16_t *p, float &x, float &y) {
+    const unsigned u = *(const unsigned *)p;
+    x = __uint_as_float(u << 16); y = __uint_as_float(u & 0xffff0000u);
+  }
+};
+template <> struct Ld<float> {
+  static __device__ __forceinline__ void v8(const float *p, float *o) {
+    const float4 x = *(const float4 *)p, y = *(const float4 *)(p + 4);
+    o[0] = x.x; o[1] = x.y; o[2] = x.z; o[3] = x.w; o[4] = y.x; o[5] = y.y; o[6] = y.z; o[7] = y.w;
+  }
+  static __device__ __forceinline__ void v2(const float *p, float &x, float &y) { const float2 v = *(const float2 *)p; x = v.x; y = v.y; }
+};
+// DVC: 128-wide pieces of the value size (a lane owns the dimension pair 2 lane, 2 lane + 1 of every piece).  VEC: key size a multiple of 8 and value size even: whole
+// key rows in 16-byte loads, value pairs in one load.
+template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) paged_window_attn_kernel(AttnArgs a) {
+  extern __shared__ float lds[];  // q [D] | p [64] | key row index [64]
+  float *qs = lds, *ps = lds + ((a.D + 3) & ~3);
+  long long *rowbase = (long long *)(ps + 64);
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int s = a.tok_seq[t], i = a.tok_pos[t], g = h / (a.H / a.G);
   const T *q = (const T *)a.q + ((size_t)t * a.H + h) * a.D;
@@ -284,9 +351,9 @@ template <class T, int DVC> __global__ void __launch_bounds__(64) paged_window_a
   int n1 = a.keep_first < w_lo ? a.keep_first : w_lo;  // kept first tokens that the window does not already cover
   if (n1 < 0) n1 = 0;
   const int total = n1 + (i - w_lo + 1);
-  float m = -FLT_MAX, l = 0.f, o[DVC];
+  float m = -FLT_MAX, l = 0.f, o[DVC][2];
 #pragma unroll
-  for (int c = 0; c < DVC; ++c) o[c] = 0.f;
+  for (int c = 0; c < DVC; ++c) o[c][0] = o[c][1] = 0.f;
   MRS_WAVE_SYNC();
   for (int v0 = 0; v0 < total; v0 += 64) {
     const int vi = v0 + lane;
@@ -297,7 +364,17 @@ template <class T, int DVC> __global__ void __launch_bounds__(64) paged_window_a
       base = ((long long)bt[key / a.block_size] * a.G + g) * a.block_size + key % a.block_size;
       const T *kr = (const T *)a.k_cache + (size_t)base * a.D;
       float acc = 0.f;
-      for (int d = 0; d < a.D; ++d) acc = fmaf(qs[d], to_f<T>(kr[d]), acc);
+      if (VEC) {
+        for (int d = 0; d < a.D; d += 8) {
+          float kv[8];
+          Ld<T>::v8(kr + d, kv);
+          const float4 qa = *(const float4 *)(qs + d), qb = *(const float4 *)(qs + d + 4);
+          acc = fmaf(qa.x, kv[0], acc); acc = fmaf(qa.y, kv[1], acc); acc = fmaf(qa.z, kv[2], acc); acc = fmaf(qa.w, kv[3], acc);
+          acc = fmaf(qb.x, kv[4], acc); acc = fmaf(qb.y, kv[5], acc); acc = fmaf(qb.z, kv[6], acc); acc = fmaf(qb.w, kv[7], acc);
+        }
+      } else {
+        for (int d = 0; d < a.D; ++d) acc = fmaf(qs[d], to_f<T>(kr[d]), acc);
+      }
       sc = acc * a.scale;
     }
     const float mn = fmaxf(m, wave_max(sc));
@@ -312,34 +389,61 @@ template <class T, int DVC> __global__ void __launch_bounds__(64) paged_window_a
     const int cnt = total - v0 < 64 ? total - v0 : 64;
 #pragma unroll
     for (int c = 0; c < DVC; ++c) {
-      const int d = lane + 64 * c;
-      float acc = o[c] * alpha;
-      if (d < a.Dv)
-        for (int j = 0; j < cnt; ++j) acc = fmaf(ps[j], to_f<T>(((const T *)a.v_cache)[(size_t)rowbase[j] * a.Dv + d]), acc);
-      o[c] = acc;
+      const int d = 128 * c + 2 * lane;
+      float a0 = o[c][0] * alpha, a1 = o[c][1] * alpha;
+      if (d < a.Dv) {
+        const T *vb = (const T *)a.v_cache + d;
+        if (VEC) {
+#pragma unroll 4
+          for (int j = 0; j < cnt; ++j) {
+            float x, y;
+            Ld<T>::v2(vb + (size_t)rowbase[j] * a.Dv, x, y);
+            a0 = fmaf(ps[j], x, a0);
+            a1 = fmaf(ps[j], y, a1);
+          }
+        } else {
+          const bool two = d + 1 < a.Dv;
+          for (int j = 0; j < cnt; ++j) {
+            const T *vr = vb + (size_t)rowbase[j] * a.Dv;
+            a0 = fmaf(ps[j], to_f<T>(vr[0]), a0);
+            if (two) a1 = fmaf(ps[j], to_f<T>(vr[1]), a1);
+          }
+        }
+      }
+      o[c][0] = a0; o[c][1] = a1;
     }
   }
   const float inv = 1.0f / l;
   T *out = (T *)a.out + ((size_t)t * a.H + h) * a.Dv;
 #pragma unroll
   for (int c = 0; c < DVC; ++c) {
-    const int d = lane + 64 * c;
-    if (d < a.Dv) out[d] = from_f<T>(o[c] * inv);
+    const int d = 128 * c + 2 * lane;
+    if (d < a.Dv) out[d] = from_f<T>(o[c][0] * inv);
+    if (d + 1 < a.Dv) out[d + 1] = from_f<T>(o[c][1] * inv);
   }
 }
 
 // ---------------------------------------------------------------------------------- mixture of experts: routing, dispatch, gather, GLU, combine
 // Router: one workgroup per row.  logits z_e = w_e . h in f32 (a wave per expert, lanes over the width, butterfly sum), score = sigmoid(z); the `top` largest (ties: the
 // lower index), weights = the scores, un-renormalised; row E of the weight (when has_gate) is the shared expert's gate: gate[t] = sigmoid(w_E . h).
-__global__ void __launch_bounds__(256) route_sigmoid_topk_kernel(const float *__restrict__ h, const float *__restrict__ wr, int W, int E, int top, int has_gate, int *__restrict__ ids,
-                                                                 float *__restrict__ wts, float *__restrict__ gate) {
+__global__ void __launch_bounds__(1024) route_sigmoid_topk_kernel(const float *__restrict__ h, const float *__restrict__ wr, int W, int E, int top, int has_gate, int *__restrict__ ids,
+                                                                  float *__restrict__ wts, float *__restrict__ gate) {
   extern __shared__ float z[];  // [E + 1]
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float *hr = h + (size_t)t * W;
-  for (int e = wave; e < E + (has_gate ? 1 : 0); e += 4) {
+  const bool vec = (W & 3) == 0;
+  for (int e = wave; e < E + (has_gate ? 1 : 0); e += 16) {
     const float *w = wr + (size_t)e * W;
     float acc = 0.f;
-    for (int k = lane; k < W; k += 64) acc = fmaf(hr[k], w[k], acc);
+    if (vec) {
+#pragma unroll 4
+      for (int k = lane * 4; k < W; k += 256) {
+        const float4 x4 = *(const float4 *)(hr + k), w4 = *(const float4 *)(w + k);
+        acc = fmaf(x4.x, w4.x, acc); acc = fmaf(x4.y, w4.y, acc); acc = fmaf(x4.z, w4.z, acc); acc = fmaf(x4.w, w4.w, acc);
+      }
+    } else {
+      for (int k = lane; k < W; k += 64) acc = fmaf(hr[k], w[k], acc);
+    }
     acc = wave_sum(acc);
     if (lane == 0) z[e] = acc;
   }
@@ -477,24 +581,34 @@ extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const
   return ok_or("mrs_hyb_conv_silu");
 }
 
-/* steps: scratch [rows, heads, 2] f32 */
-extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, float *state, float *out, const int *seq_start,
-                                const int *seq_pos0, const int *seq_slot, float *steps, int rows, int entries, int C, int ldu, int dt_col, int heads, int P, int N, int G,
-                                void *stream) {
-  if (entries <= 0 || rows <= 0) return 0;
+/* steps: scratch [rows, heads, 2] f32.  Segment table (host-built): seg_entry / seg_row0 / seg_len [segments], ent_seg0 [entries + 1]; carry [segments, heads, N, P] and
+ * decay [segments, heads] are scratch that is only touched when some entry has more than one segment (segments > entries). */
+extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, float *state, float *out, const int *seq_pos0,
+                                const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry,
+                                float *decay, int rows, int entries, int segments, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream) {
+  if (entries <= 0 || rows <= 0 || segments <= 0) return 0;
   if (heads <= 0 || G <= 0 || heads % G || P <= 0 || N <= 0) return fail("mrs_hyb_ssd_scan: bad head / group sizes");
-  ScanArgs a{xbc, u, dt_bias, A_log, D, steps, state, out, seq_start, seq_pos0, seq_slot, C, ldu, dt_col, heads, P, N, G, rows};
+  if (segments > 65535 || entries > 65535) return fail("mrs_hyb_ssd_scan: more than 65535 segments in one step");
+  if (segments > entries && (!carry || !decay)) return fail("mrs_hyb_ssd_scan: segmented entries need the carry scratch");
+  ScanArgs a{xbc, u, dt_bias, A_log, D, steps, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, decay, C, ldu, dt_col, heads, P, N, G, rows};
   hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
   const bool vec = C % 4 == 0 && (heads * P) % 4 == 0 && N % 4 == 0 && ((uintptr_t)xbc % 16) == 0;
-#define MRS_SCAN(R, K) do { if (vec) hipLaunchKernelGGL((ssd_scan_kernel<R, K, true>), dim3((P + 64 / R - 1) / (64 / R), heads, entries), dim3(64), 0, S_(stream), a); \
-                            else hipLaunchKernelGGL((ssd_scan_kernel<R, K, false>), dim3((P + 64 / R - 1) / (64 / R), heads, entries), dim3(64), 0, S_(stream), a); } while (0)
-  if (N <= 16) MRS_SCAN(2, 8);
-  else if (N <= 64) MRS_SCAN(4, 16);
-  else if (N <= 128) MRS_SCAN(4, 32);
-  else if (N <= 256) MRS_SCAN(8, 32);
-  else if (N <= 512) MRS_SCAN(16, 32);
+  const bool single = rows == segments;  // one row per segment (decode steps): no ring
+  const bool split = segments > entries;
+#define MRS_SCAN_(R, K, V, DP, L) hipLaunchKernelGGL((ssd_scan_kernel<R, K, V, DP, L>), dim3((P + 64 / R - 1) / (64 / R), heads, segments), dim3(64), 0, S_(stream), a)
+#define MRS_SCAN(R, K, DP) do { \
+    if (split) { if (vec) MRS_SCAN_(R, K, true, DP, true); else MRS_SCAN_(R, K, false, DP, true); \
+                 hipLaunchKernelGGL(ssd_carry_kernel, dim3((N * P + 255) / 256, heads, entries), dim3(256), 0, S_(stream), a); } \
+    if (single) { if (vec) MRS_SCAN_(R, K, true, 1, false); else MRS_SCAN_(R, K, false, 1, false); } \
+    else { if (vec) MRS_SCAN_(R, K, true, DP, false); else MRS_SCAN_(R, K, false, DP, false); } } while (0)
+  if (N <= 16) MRS_SCAN(2, 8, 8);
+  else if (N <= 64) MRS_SCAN(4, 16, 6);
+  else if (N <= 128) MRS_SCAN(4, 32, 4);
+  else if (N <= 256) MRS_SCAN(8, 32, 4);
+  else if (N <= 512) MRS_SCAN(16, 32, 4);
   else return fail("mrs_hyb_ssd_scan: state size above 512");
 #undef MRS_SCAN
+#undef MRS_SCAN_
   return ok_or("mrs_hyb_ssd_scan");
 }
 
@@ -515,12 +629,14 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
   if (rows <= 0) return 0;
   if (Dv > 256 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 256 / heads % kv_heads");
   AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale};
-  const size_t lds = (size_t)(D + 64 + 2) * 4 + 64 * 8;
+  const size_t lds = (size_t)(((D + 3) & ~3) + 64) * 4 + 64 * 8;
   dim3 grid(rows, H);
-#define MRS_ATTN(T, C) hipLaunchKernelGGL((paged_window_attn_kernel<T, C>), grid, dim3(64), lds, S_(stream), a)
-  const int c = (Dv + 63) / 64;
-  if (dtype == 1) { if (c <= 1) MRS_ATTN(mrs::bf16_t, 1); else if (c <= 2) MRS_ATTN(mrs::bf16_t, 2); else MRS_ATTN(mrs::bf16_t, 4); }
-  else if (dtype == 2) { if (c <= 1) MRS_ATTN(float, 1); else if (c <= 2) MRS_ATTN(float, 2); else MRS_ATTN(float, 4); }
+  const bool vec = D % 8 == 0 && Dv % 2 == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 8) == 0;
+#define MRS_ATTN(T, C) do { if (vec) hipLaunchKernelGGL((paged_window_attn_kernel<T, C, true>), grid, dim3(64), lds, S_(stream), a); \
+                            else hipLaunchKernelGGL((paged_window_attn_kernel<T, C, false>), grid, dim3(64), lds, S_(stream), a); } while (0)
+  const int c = (Dv + 127) / 128;
+  if (dtype == 1) { if (c <= 1) MRS_ATTN(mrs::bf16_t, 1); else MRS_ATTN(mrs::bf16_t, 2); }
+  else if (dtype == 2) { if (c <= 1) MRS_ATTN(float, 1); else MRS_ATTN(float, 2); }
   else return fail("mrs_hyb_paged_window_attn: dtype");
 #undef MRS_ATTN
   return ok_or("mrs_hyb_paged_window_attn");
@@ -530,7 +646,7 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
 extern "C" int mrs_hyb_route_sigmoid_topk(const float *h, const float *wr, int rows, int W, int E, int top, int has_gate, int *ids, float *wts, float *gate, void *stream) {
   if (rows <= 0) return 0;
   if (top < 1 || top > E || E > 8192) return fail("mrs_hyb_route_sigmoid_topk: 1 <= top <= experts <= 8192");
-  hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3(rows), dim3(256), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, has_gate, ids, wts, gate);
+  hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, has_gate, ids, wts, gate);
   return ok_or("mrs_hyb_route_sigmoid_topk");
 }
 

@@ -32,7 +32,7 @@ _SIGS = {
     "mrs_hyb_embed": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "mrs_hyb_rmsnorm": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _i, _vp],
     "mrs_hyb_conv_silu": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
-    "mrs_hyb_ssd_scan": [_vp] * 11 + [_i] * 10 + [_vp],
+    "mrs_hyb_ssd_scan": [_vp] * 16 + [_i] * 10 + [_vp],
     "mrs_hyb_qk_norm_rope_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "mrs_hyb_paged_window_attn": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp],
     "mrs_hyb_route_sigmoid_topk": [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp],
@@ -74,6 +74,14 @@ class RaggedBatch:
     block_tables: torch.Tensor  # i32 [entries, max_blocks]
     slot_mapping: torch.Tensor  # i64 [rows]  K / V page slot = block * block_size + offset
     want: torch.Tensor          # i32 [n]  rows whose logits are wanted
+    # every entry's rows cut into segments of at most SEGMENT rows (linear recurrences run the segments of a long portion in parallel)
+    segments: int = 0
+    seg_entry: Optional[torch.Tensor] = None   # i32 [segments]
+    seg_row0: Optional[torch.Tensor] = None    # i32 [segments]  first row
+    seg_len: Optional[torch.Tensor] = None     # i32 [segments]
+    ent_seg0: Optional[torch.Tensor] = None    # i32 [entries + 1]  first segment of every entry, then the total
+
+    SEGMENT = 128
 
     @staticmethod
     def build(entries: Sequence[dict], block_size: int, device) -> "RaggedBatch":
@@ -82,13 +90,17 @@ class RaggedBatch:
         lens = [len(e["tokens"]) for e in entries]
         T = sum(lens)
         mb = max(1, max((len(e["blocks"]) for e in entries), default=1))
-        ints = np.zeros(3 * T + (S + 1) + 2 * S + S * mb, dtype=np.int32)
+        L = RaggedBatch.SEGMENT
+        nseg = sum(max(1, -(-n // L)) for n in lens)
+        sizes = (T, T, T, S + 1, S, S, S * mb, nseg, nseg, nseg, S + 1)
+        ints = np.zeros(sum(sizes), dtype=np.int32)
         o = 0
         views = []
-        for n in (T, T, T, S + 1, S, S, S * mb):
+        for n in sizes:
             views.append(ints[o:o + n])
             o += n
-        tok, tseq, tpos, sst, sp0, ssl, bt = views
+        tok, tseq, tpos, sst, sp0, ssl, bt, sge, sgr, sgl, es0 = views
+        z = 0
         bt = bt.reshape(S, mb)
         slots = np.zeros(T, dtype=np.int64)
         want: List[int] = []
@@ -109,16 +121,21 @@ class RaggedBatch:
             if n:
                 slots[r:r + n] = blocks[pos // block_size] * block_size + pos % block_size
             want.extend(r + int(j) for j in e.get("want", ()))
+            es0[s] = z
+            for a0 in range(0, max(n, 1), L):
+                sge[z], sgr[z], sgl[z] = s, r + a0, min(L, n - a0)
+                z += 1
             r += n
         sst[S] = T
+        es0[S] = z
         dev_ints = torch.from_numpy(ints).to(device)
         o = 0
         dv = []
-        for n in (T, T, T, S + 1, S, S, S * mb):
+        for n in sizes:
             dv.append(dev_ints[o:o + n])
             o += n
         return RaggedBatch(T, S, mb, dv[0], dv[1], dv[2], dv[3], dv[4], dv[5], dv[6].view(S, mb), torch.from_numpy(slots).to(device),
-                           torch.tensor(want, dtype=torch.int32, device=device))
+                           torch.tensor(want, dtype=torch.int32, device=device), nseg, dv[7], dv[8], dv[9], dv[10])
 
 
 # ------------------------------------------------------------------------------------------------------------------ layer descriptions
@@ -268,8 +285,12 @@ class Mamba2Mixer(_Module):
               T, b.entries, s.conv_channels, s.conv)
         y = torch.empty(T, s.inner, dtype=torch.float32, device=m.device)
         steps = torch.empty(T, s.heads, 2, dtype=torch.float32, device=m.device)
-        _call("mrs_hyb_ssd_scan", xbc, u, self.dt_bias, self.A_log, self.D, self.ssm_state, y, b.seq_start, b.seq_pos0, b.seq_slot, steps, T, b.entries, s.conv_channels,
-              u.stride(0), s.inner + s.conv_channels, s.heads, s.vdim, s.state, s.groups)
+        carry = decay = None
+        if b.segments > b.entries:   # some portion is longer than a segment: scratch for the segments' local end states
+            carry = torch.empty(b.segments, s.heads, s.state, s.vdim, dtype=torch.float32, device=m.device)
+            decay = torch.empty(b.segments, s.heads, dtype=torch.float32, device=m.device)
+        _call("mrs_hyb_ssd_scan", xbc, u, self.dt_bias, self.A_log, self.D, self.ssm_state, y, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0,
+              steps, carry, decay, T, b.entries, b.segments, s.conv_channels, u.stride(0), s.inner + s.conv_channels, s.heads, s.vdim, s.state, s.groups)
         yn = m.norm(y, self.norm, one_plus=False, parts=s.norm_groups, gate=u)   # y * silu(z) (z = the first `inner` columns of u), then the grouped norm
         m.linear(yn, self.w_o, out=x, accumulate=True)
 
@@ -510,7 +531,9 @@ class DecodeGraph:
         for k in (n, n, n, n + 1, n, n, n * mb):
             v.append(self._ints[o:o + k])
             o += k
-        self.batch = RaggedBatch(n, n, mb, v[0], v[1], v[2], v[3], v[4], v[5], v[6].view(n, mb), self._slots, torch.arange(n, dtype=torch.int32, device=dev))
+        rows = torch.arange(n + 1, dtype=torch.int32, device=dev)   # one row = one segment per entry
+        self.batch = RaggedBatch(n, n, mb, v[0], v[1], v[2], v[3], v[4], v[5], v[6].view(n, mb), self._slots, rows[:n].clone(), n, rows[:n], rows[:n],
+                                 torch.ones(n, dtype=torch.int32, device=dev), rows)
         self._host = np.zeros(self._ints.numel(), dtype=np.int32)
         self._host[3 * n:3 * n + n + 1] = np.arange(n + 1)          # seq_start: one row per entry
         self._host[2 * n:3 * n] = 1                                  # positions >= 1 during warm-up: the slots' states are read, nothing is reset
