@@ -95,8 +95,8 @@ __global__ void __launch_bounds__(256) gemm_tile_bf16_kernel(GemmArgs a) {
     for (int ks = 0; ks < BK; ks += 16) {
       const bf16x8 af = __builtin_bit_cast(bf16x8, *(const int4 *)&As[wm + ql][ks + 8 * kh]);
       const bf16x8 wf = __builtin_bit_cast(bf16x8, *(const int4 *)&Ws[wn + ql][ks + 8 * kh]);
-      // D[i][j] = sum_k X[i][k] Y[k][j]: X = weights (i = output column n), Y = activations (j = row m): a lane then holds 16 n for ONE m... the other way round
-      // keeps stores coalesced: X = activations (i = m), Y = weights (j = n); lane (ql, kh) ends up with column n = ql and rows (r & 3) + 8 (r >> 2) + 4 kh
+      // D[i][j] = sum_k X[i][k] Y[k][j] with X = activations (i = row m) and Y = weights (j = column n): lane (ql, kh) ends up with column n = ql and the rows
+      // (r & 3) + 8 (r >> 2) + 4 kh, so the stores of a register are 32 consecutive floats of one output row
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, wf, acc, 0, 0, 0);
     }
     __syncthreads();
@@ -171,6 +171,11 @@ __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
 }
 
 // ---------------------------------------------------------------------------------- M <= 8 rows
+// The activation operand of a row kernel can be produced on the fly (decode steps: one launch less per use):
+//   IN_PLAIN   A [M, K] in T
+//   IN_GLU     A = f32 [M, 2 K] = gate | up of the previous product: x_k = round_T(silu(gate_k) * up_k)
+//   IN_SCALED  A = f32 [rows, K] normed rows: row m reads source row src_row[m] / src_div times src_scale[src_row[m]], rounded to T (expert-sorted routed inputs)
+enum { IN_PLAIN = 0, IN_GLU = 1, IN_SCALED = 2 };
 struct GemvArgs {
   const void *A;
   const void *W;
@@ -180,6 +185,9 @@ struct GemvArgs {
   const int *row_group;      // grouped: row m multiplies W + row_group[m] * wstride (grid.y = M, one row per workgroup row), else null
   long long wstride;
   int vec_ok;
+  const int *src_row;        // IN_SCALED
+  const float *src_scale;
+  int src_div;
 };
 
 template <class T> struct Vec8;
@@ -204,12 +212,38 @@ template <> struct Vec8<float> {
   }
   static __device__ __forceinline__ void load_nt(const float *p, float *o) { load(p, o); }
 };
+__device__ __forceinline__ float silu_in(float v) { return v / (1.0f + expf(-v)); }
 
-template <class T, int MR> __global__ void __launch_bounds__(256) gemv_rows_kernel(GemvArgs a) {
+// one activation value (element path) / eight (vector path) of row m at column k, as the product sees it
+template <class T, int IN> __device__ __forceinline__ float act1(const GemvArgs &a, int m, int k) {
+  if (IN == IN_PLAIN) return to_f<T>(((const T *)a.A)[(size_t)m * a.lda + k]);
+  const float *A = (const float *)a.A;
+  if (IN == IN_GLU) return round_to<T>(silu_in(A[(size_t)m * a.lda + k]) * A[(size_t)m * a.lda + a.K + k]);
+  const int r = a.src_row[m];
+  return round_to<T>(a.src_scale[r] * A[(size_t)(r / a.src_div) * a.lda + k]);
+}
+template <class T, int IN> __device__ __forceinline__ void act8(const GemvArgs &a, int m, int k, float *x) {
+  if (IN == IN_PLAIN) { Vec8<T>::load((const T *)a.A + (size_t)m * a.lda + k, x); return; }
+  const float *A = (const float *)a.A;
+  if (IN == IN_GLU) {
+    float g[8], u[8];
+    Vec8<float>::load(A + (size_t)m * a.lda + k, g);
+    Vec8<float>::load(A + (size_t)m * a.lda + a.K + k, u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = round_to<T>(silu_in(g[j]) * u[j]);
+    return;
+  }
+  const int r = a.src_row[m];
+  const float w = a.src_scale[r];
+  Vec8<float>::load(A + (size_t)(r / a.src_div) * a.lda + k, x);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) x[j] = round_to<T>(w * x[j]);
+}
+
+template <class T, int MR, int IN> __global__ void __launch_bounds__(256) gemv_rows_kernel(GemvArgs a) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int n = blockIdx.x * 4 + wave;
   if (n >= a.N) return;
-  const T *A = (const T *)a.A;
   const T *W = (const T *)a.W;
   int m_lo = 0, m_cnt = a.M;
   if (a.row_group) {
@@ -228,7 +262,7 @@ template <class T, int MR> __global__ void __launch_bounds__(256) gemv_rows_kern
 #pragma unroll
       for (int m = 0; m < MR; ++m)
         if (m < m_cnt) {
-          Vec8<T>::load(A + (size_t)(m_lo + m) * a.lda + k, x);
+          act8<T, IN>(a, m_lo + m, k, x);
 #pragma unroll
           for (int j = 0; j < 8; ++j) acc[m] = fmaf(w[j], x[j], acc[m]);
         }
@@ -238,7 +272,7 @@ template <class T, int MR> __global__ void __launch_bounds__(256) gemv_rows_kern
       const float w = to_f<T>(wr[k]);
 #pragma unroll
       for (int m = 0; m < MR; ++m)
-        if (m < m_cnt) acc[m] = fmaf(w, to_f<T>(A[(size_t)(m_lo + m) * a.lda + k]), acc[m]);
+        if (m < m_cnt) acc[m] = fmaf(w, act1<T, IN>(a, m_lo + m, k), acc[m]);
     }
   }
 #pragma unroll
@@ -279,21 +313,26 @@ extern "C" int mrs_hyb_gemm(const void *A, const void *W, float *C, int M, int N
   return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemm: launch failed");
 }
 
+/* in_mode: 0 plain (A in dtype), 1 GLU (A = f32 [M, 2 K] gate | up), 2 scaled rows (A = f32 source rows; row m = src_scale[r] * A[r / src_div], r = src_row[m]) */
 extern "C" int mrs_hyb_gemv(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
-                            const int *row_group, long long wstride, void *stream) {
+                            const int *row_group, long long wstride, int in_mode, const int *src_row, const float *src_scale, int src_div, void *stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2)) return fail("mrs_hyb_gemv: bad shape / dtype");
+  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2) || in_mode < 0 || in_mode > 2) return fail("mrs_hyb_gemv: bad shape / dtype / input mode");
+  if (in_mode == 1 && lda < 2 * K) return fail("mrs_hyb_gemv: the gate | up operand needs rows of 2 K values");
+  if (in_mode == 2 && (!src_row || !src_scale || src_div <= 0)) return fail("mrs_hyb_gemv: scaled rows need their source table");
   if (!row_group && M > 8) return fail("mrs_hyb_gemv: at most 8 rows share a weight");
   if (row_group && M > 65535) return fail("mrs_hyb_gemv: too many rows");
   const int esz = dtype == 1 ? 2 : 4;
   GemvArgs a{A, W, C, M, N, K, lda, ldw, ldc, accumulate, row_group, wstride,
-             (K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0) ? 1 : 0};
+             (K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0) ? 1 : 0, src_row, src_scale, src_div};
   dim3 grid((N + 3) / 4, row_group ? M : 1);
   hipStream_t s = (hipStream_t)stream;
-#define MRS_GEMV(T, MR) hipLaunchKernelGGL((gemv_rows_kernel<T, MR>), grid, dim3(256), 0, s, a)
+#define MRS_GEMV_(T, MR, IN) hipLaunchKernelGGL((gemv_rows_kernel<T, MR, IN>), grid, dim3(256), 0, s, a)
+#define MRS_GEMV(T, MR) do { if (in_mode == 0) MRS_GEMV_(T, MR, IN_PLAIN); else if (in_mode == 1) MRS_GEMV_(T, MR, IN_GLU); else MRS_GEMV_(T, MR, IN_SCALED); } while (0)
   const int mr = row_group ? 1 : M;
   if (dtype == 1) { if (mr <= 1) MRS_GEMV(mrs::bf16_t, 1); else if (mr <= 2) MRS_GEMV(mrs::bf16_t, 2); else if (mr <= 4) MRS_GEMV(mrs::bf16_t, 4); else MRS_GEMV(mrs::bf16_t, 8); }
   else { if (mr <= 1) MRS_GEMV(float, 1); else if (mr <= 2) MRS_GEMV(float, 2); else if (mr <= 4) MRS_GEMV(float, 4); else MRS_GEMV(float, 8); }
 #undef MRS_GEMV
+#undef MRS_GEMV_
   return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemv: launch failed");
 }

@@ -88,6 +88,32 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const float *__restrict_
   }
   out[(size_t)t * C + c] = silu_f(acc);
 }
+// decode steps (every entry brings one row): convolution and tap shift in one launch, the thread of (entry, channel) reads its taps, then writes them
+__global__ void __launch_bounds__(256) conv_silu_step_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ cw, const float *__restrict__ cb, float *__restrict__ state,
+                                                             const int *__restrict__ seq_start, const int *__restrict__ seq_pos0, const int *__restrict__ seq_slot,
+                                                             float *__restrict__ out, int C, int taps) {
+  const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int row = seq_start[s], keep = taps - 1;
+  if (seq_start[s + 1] - row != 1) return;
+  const bool carried = seq_pos0[s] > 0;
+  float *st = state + ((size_t)seq_slot[s] * C + c) * keep;
+  const float cur = u[(size_t)row * ldu + c];
+  float acc = cb[c], v[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    if (k >= keep) break;
+    v[k] = carried ? st[k] : 0.f;
+    acc = fmaf(cw[(size_t)c * taps + k], v[k], acc);
+  }
+  acc = fmaf(cw[(size_t)c * taps + keep], cur, acc);
+  out[(size_t)row * C + c] = silu_f(acc);
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    if (k >= keep) break;
+    st[k] = k + 1 < keep ? v[k + 1] : cur;
+  }
+}
 // the slot's taps after the step: the last taps - 1 inputs of (old taps ++ this step's rows).  One thread per (entry, channel) reads everything before it writes.
 __global__ void __launch_bounds__(256) conv_state_kernel(const float *__restrict__ u, int ldu, float *__restrict__ state, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
                                                          const int *__restrict__ seq_slot, int C, int taps) {
@@ -204,8 +230,14 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
       }
     }
     g_.x = xr[h * a.P + pc];
-    const float *de = a.steps + 2 * ((size_t)row * a.heads + h);
-    const float d0 = de[0], d1 = de[1];
+    float d0, d1;
+    if (DEPTH == 1 && !LOCAL) {  // decode steps: the step size and decay inline (ssd_steps_kernel's expressions), one launch less
+      d0 = softplus_f(a.u[(size_t)row * a.ldu + a.dt_col + h] + a.dt_bias[h]);
+      d1 = expf(-expf(a.A_log[h]) * d0);
+    } else {
+      const float *de = a.steps + 2 * ((size_t)row * a.heads + h);
+      d0 = de[0]; d1 = de[1];
+    }
     g_.dt = i < len ? d0 : 0.f;    // past the end: S <- 1 S + 0
     g_.dec = i < len ? d1 : 1.f;
   };
@@ -575,6 +607,10 @@ extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const
                                  const int *seq_slot, float *out, int rows, int entries, int C, int taps, void *stream) {
   if (rows <= 0) return 0;
   if (taps < 1 || taps > 17) return fail("mrs_hyb_conv_silu: 1 .. 17 taps");
+  if (rows == entries) {  // one row per entry (an entry without rows cannot occur then)
+    hipLaunchKernelGGL(conv_silu_step_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, cw, cb, state, seq_start, seq_pos0, seq_slot, out, C, taps);
+    return ok_or("mrs_hyb_conv_silu");
+  }
   hipLaunchKernelGGL(conv_silu_kernel, dim3(rows, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps);
   if (taps > 1)
     hipLaunchKernelGGL(conv_state_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, state, seq_start, seq_pos0, seq_slot, C, taps);
@@ -591,9 +627,9 @@ extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *d
   if (segments > 65535 || entries > 65535) return fail("mrs_hyb_ssd_scan: more than 65535 segments in one step");
   if (segments > entries && (!carry || !decay)) return fail("mrs_hyb_ssd_scan: segmented entries need the carry scratch");
   ScanArgs a{xbc, u, dt_bias, A_log, D, steps, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, decay, C, ldu, dt_col, heads, P, N, G, rows};
-  hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
   const bool vec = C % 4 == 0 && (heads * P) % 4 == 0 && N % 4 == 0 && ((uintptr_t)xbc % 16) == 0;
-  const bool single = rows == segments;  // one row per segment (decode steps): no ring
+  const bool single = rows == segments;  // one row per segment (decode steps): no ring, step sizes inline
+  if (!single) hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
   const bool split = segments > entries;
 #define MRS_SCAN_(R, K, V, DP, L) hipLaunchKernelGGL((ssd_scan_kernel<R, K, V, DP, L>), dim3((P + 64 / R - 1) / (64 / R), heads, segments), dim3(64), 0, S_(stream), a)
 #define MRS_SCAN(R, K, DP) do { \

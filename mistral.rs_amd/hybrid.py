@@ -42,7 +42,7 @@ _SIGS = {
     "mrs_hyb_moe_combine": [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp],
     "mrs_hyb_gather_rows": [_vp, _vp, _vp, _i, _i, _vp],
     "mrs_hyb_gemm": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _l, _i, _vp],
-    "mrs_hyb_gemv": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _vp],
+    "mrs_hyb_gemv": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp],
 }
 _fns: dict = {}
 
@@ -367,18 +367,30 @@ class SigmoidMoe(_Module):
         meta = torch.empty(s.experts + 1 + 3 * R, dtype=torch.int32, device=dev)
         bounds, sorted_route, route_pos, sorted_expert = meta[:s.experts + 1], meta[s.experts + 1:][:R], meta[s.experts + 1 + R:][:R], meta[s.experts + 1 + 2 * R:][:R]
         _call("mrs_hyb_moe_dispatch", ids, R, s.experts, bounds, sorted_route, route_pos, sorted_expert)
-        xs = torch.empty(R, W, dtype=m.torch_dtype, device=dev)
-        _call("mrs_hyb_moe_gather", h32, sorted_route, wts, s.top, xs, R, W, m.dt)
-        gu = m.grouped_linear(xs, self.w_gu, bounds, sorted_expert)
-        act = torch.empty(R, s.ff, dtype=m.torch_dtype, device=dev)
-        _call("mrs_hyb_glu_silu", gu, act, R, s.ff, m.dt)
-        d = m.grouped_linear(act, self.w_down, bounds, sorted_expert)
+        f32 = dict(dtype=torch.float32, device=dev)
+        if R <= m.GROUPED_GEMV_ROWS:
+            # decode-sized steps: every route streams its expert's slabs; the scaled gather and the GLU happen in the consuming product's operand load (same roundings)
+            gu = torch.empty(R, 2 * s.ff, **f32)
+            _call("mrs_hyb_gemv", h32, self.w_gu, gu, R, 2 * s.ff, W, h32.stride(0), W, 2 * s.ff, m.dt, 0, sorted_expert, self.w_gu.stride(0), 2, sorted_route, wts, s.top)
+            d = torch.empty(R, W, **f32)
+            _call("mrs_hyb_gemv", gu, self.w_down, d, R, W, s.ff, 2 * s.ff, s.ff, W, m.dt, 0, sorted_expert, self.w_down.stride(0), 1, None, None, 1)
+        else:
+            xs = torch.empty(R, W, dtype=m.torch_dtype, device=dev)
+            _call("mrs_hyb_moe_gather", h32, sorted_route, wts, s.top, xs, R, W, m.dt)
+            gu = m.grouped_linear(xs, self.w_gu, bounds, sorted_expert)
+            act = torch.empty(R, s.ff, dtype=m.torch_dtype, device=dev)
+            _call("mrs_hyb_glu_silu", gu, act, R, s.ff, m.dt)
+            d = m.grouped_linear(act, self.w_down, bounds, sorted_expert)
         sh = None
         if s.shared_ff:
             sgu = m.linear(h, self.ws_gu)
-            sact = torch.empty(T, s.shared_ff, dtype=m.torch_dtype, device=dev)
-            _call("mrs_hyb_glu_silu", sgu, sact, T, s.shared_ff, m.dt)
-            sh = m.linear(sact, self.ws_down)
+            if T <= m.GEMV_ROWS:
+                sh = torch.empty(T, W, **f32)
+                _call("mrs_hyb_gemv", sgu, self.ws_down, sh, T, W, s.shared_ff, 2 * s.shared_ff, s.shared_ff, W, m.dt, 0, None, 0, 1, None, None, 1)
+            else:
+                sact = torch.empty(T, s.shared_ff, dtype=m.torch_dtype, device=dev)
+                _call("mrs_hyb_glu_silu", sgu, sact, T, s.shared_ff, m.dt)
+                sh = m.linear(sact, self.ws_down)
         _call("mrs_hyb_moe_combine", x, d, route_pos, s.top, sh, gate, T, W)
 
 
@@ -464,7 +476,7 @@ class HybridDecoder:
             out = torch.empty(M, N, dtype=torch.float32, device=self.device)
         dt = dtype_code or self.dt
         if M <= self.GEMV_ROWS:
-            _call("mrs_hyb_gemv", a, w, out, M, N, K, a.stride(0), w.stride(0), out.stride(0), dt, int(accumulate), None, 0)
+            _call("mrs_hyb_gemv", a, w, out, M, N, K, a.stride(0), w.stride(0), out.stride(0), dt, int(accumulate), None, 0, 0, None, None, 1)
         else:
             _call("mrs_hyb_gemm", a, w, out, M, N, K, a.stride(0), w.stride(0), out.stride(0), dt, int(accumulate), None, 0, 0, 0)
         return out
@@ -475,7 +487,7 @@ class HybridDecoder:
         E, N = w.shape[0], w.shape[1]
         out = torch.empty(R, N, dtype=torch.float32, device=self.device)
         if R <= self.GROUPED_GEMV_ROWS:
-            _call("mrs_hyb_gemv", a, w, out, R, N, K, a.stride(0), w.stride(1), out.stride(0), self.dt, 0, sorted_expert, w.stride(0))
+            _call("mrs_hyb_gemv", a, w, out, R, N, K, a.stride(0), w.stride(1), out.stride(0), self.dt, 0, sorted_expert, w.stride(0), 0, None, None, 1)
         else:
             _call("mrs_hyb_gemm", a, w, out, R, N, K, a.stride(0), w.stride(1), out.stride(0), self.dt, 0, bounds, E, w.stride(0), R)
         return out
