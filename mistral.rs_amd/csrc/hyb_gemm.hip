@@ -114,6 +114,89 @@ __global__ void __launch_bounds__(256) gemm_tile_bf16_kernel(GemmArgs a) {
   }
 }
 
+// 128 x 128 tile for prompt-sized products: every wave owns a 64 x 64 quadrant (2 x 2 MFMA tiles: each operand fragment read from LDS feeds two MFMAs), and the next
+// K-step's global loads are in registers while the current one multiplies (one LDS buffer, two barriers per step).
+__global__ void __launch_bounds__(256) gemm_tile128_bf16_kernel(GemmArgs a) {
+  constexpr int TM = 128, TN = 128;
+  __shared__ __attribute__((aligned(16))) uint16_t As[TM][BK + 8];
+  __shared__ __attribute__((aligned(16))) uint16_t Ws[TN][BK + 8];
+  int row_lo = 0, row_hi = a.M;
+  const bf16_t *W = (const bf16_t *)a.W;
+  if (a.bounds) {
+    row_lo = a.bounds[blockIdx.z];
+    row_hi = a.bounds[blockIdx.z + 1];
+    W += (size_t)blockIdx.z * a.wstride;
+  }
+  const int m0 = row_lo + blockIdx.y * TM, n0 = blockIdx.x * TN;
+  if (m0 >= row_hi) return;
+  const bf16_t *A = (const bf16_t *)a.A;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ql = lane & 31, kh = lane >> 5;
+  const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
+  const int lr = tid >> 2, kc = (tid & 3) * 8;  // this thread stages rows lr and lr + 64 of both operands, 8 values at kc
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  auto fetch = [&](const bf16_t *base, int ld, int row, int rows_end, int k0) -> int4 {
+    int4 v = make_int4(0, 0, 0, 0);
+    if (row < rows_end) {
+      const bf16_t *p = base + (size_t)row * ld + k0 + kc;
+      if (a.vec_ok && k0 + kc + 8 <= a.K) v = *(const int4 *)p;
+      else {
+        uint16_t t[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = (k0 + kc + j < a.K) ? p[j].v : (uint16_t)0;
+        v = make_int4((int)(t[0] | ((unsigned)t[1] << 16)), (int)(t[2] | ((unsigned)t[3] << 16)), (int)(t[4] | ((unsigned)t[5] << 16)), (int)(t[6] | ((unsigned)t[7] << 16)));
+      }
+    }
+    return v;
+  };
+  int4 ra[2], rw[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) { ra[i] = fetch(A, a.lda, m0 + lr + 64 * i, row_hi, 0); rw[i] = fetch(W, a.ldw, n0 + lr + 64 * i, a.N, 0); }
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) { *(int4 *)&As[lr + 64 * i][kc] = ra[i]; *(int4 *)&Ws[lr + 64 * i][kc] = rw[i]; }
+    __syncthreads();
+    if (k0 + BK < a.K) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) { ra[i] = fetch(A, a.lda, m0 + lr + 64 * i, row_hi, k0 + BK); rw[i] = fetch(W, a.ldw, n0 + lr + 64 * i, a.N, k0 + BK); }
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 16) {
+      bf16x8 af[2], wf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        af[i] = __builtin_bit_cast(bf16x8, *(const int4 *)&As[wm + 32 * i + ql][ks + 8 * kh]);
+        wf[i] = __builtin_bit_cast(bf16x8, *(const int4 *)&Ws[wn + 32 * i + ql][ks + 8 * kh]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn + 32 * j + ql;
+    if (n >= a.N) continue;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + 32 * i + (r & 3) + 8 * (r >> 2) + 4 * kh;
+        if (m < row_hi) {
+          float *c = a.C + (size_t)m * a.ldc + n;
+          *c = a.accumulate ? *c + acc[i][j][r] : acc[i][j][r];
+        }
+      }
+  }
+}
+
 __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
   __shared__ __attribute__((aligned(16))) float As[BM][BK + 4];
   __shared__ __attribute__((aligned(16))) float Ws[BN][BK + 4];
@@ -306,6 +389,13 @@ extern "C" int mrs_hyb_gemm(const void *A, const void *W, float *C, int M, int N
              (K % vq == 0 && lda % vq == 0 && ldw % vq == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0) ? 1 : 0};
   const int rows = groups > 0 ? max_rows : M;
   if (rows <= 0) return 0;
+  // prompt-sized bf16 products take the 128 x 128 tile: dense from 256 rows, grouped when a group averages a full tile of rows
+  if (dtype == 1 && N >= 128 && (groups > 0 ? M / groups >= 128 : M >= 256)) {
+    dim3 g2((N + 127) / 128, (rows + 127) / 128, groups > 0 ? groups : 1);
+    if (g2.y > 65535 || g2.z > 65535) return fail("mrs_hyb_gemm: too many row tiles / groups for one launch");
+    hipLaunchKernelGGL(gemm_tile128_bf16_kernel, g2, dim3(256), 0, (hipStream_t)stream, a);
+    return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemm: launch failed");
+  }
   dim3 grid((N + BN - 1) / BN, (rows + BM - 1) / BM, groups > 0 ? groups : 1);
   if (grid.y > 65535 || grid.z > 65535) return fail("mrs_hyb_gemm: too many row tiles / groups for one launch");
   if (dtype == 1) hipLaunchKernelGGL(gemm_tile_bf16_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);

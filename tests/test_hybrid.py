@@ -241,7 +241,7 @@ def _batch_of(sv, n, rid=1):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N,K", [(1, 37, 40), (3, 64, 24), (8, 130, 72), (9, 65, 33), (70, 129, 96), (200, 31, 256)])
+@pytest.mark.parametrize("M,N,K", [(1, 37, 40), (3, 64, 24), (8, 130, 72), (9, 65, 33), (70, 129, 96), (200, 31, 256), (300, 260, 96), (257, 128, 41)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_linear_products(dev, M, N, K, dtype):
     """out (+)= a . w^T through the row kernel (M <= 8) and the tile kernel, odd sizes included (K = 33: the element-wise load path)"""
@@ -259,12 +259,12 @@ def test_linear_products(dev, M, N, K, dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("R", [5, 32, 33, 150])
+@pytest.mark.parametrize("R", [5, 32, 33, 150, 900])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_grouped_products(dev, R, dtype):
     """rows sorted by group, one weight slab per group; empty groups and groups larger than a tile"""
     _, _, sv = _one_layer(mamba_layer(mlp=False), dev, dtype)
-    E, N, K = 6, 50, 40
+    E, N, K = (6, 50, 40) if R < 900 else (4, 136, 72)   # 900 rows over 4 groups: the 128-row tile form
     g = torch.Generator().manual_seed(R)
     grp = torch.sort(torch.randint(0, E, (R,), generator=g)).values
     grp[grp == 2] = 3  # group 2 stays empty
