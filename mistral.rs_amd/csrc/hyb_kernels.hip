@@ -273,6 +273,111 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
       if (k < nk) st[(size_t)(r * K + k) * a.P + p] = S[k];
 }
 
+// The same recurrence for portions (segments of many rows), operands through LDS: the waves of one (segment, head) -- one per 64 / R values of P -- share the rows' B, C, x and
+// step values.  TC rows are staged at a time with coalesced loads (every value is read from global memory once per head instead of once per lane group), the next TC rows
+// are in registers while the current ones are consumed, and a lane reads its K state rows' B / C as broadcast 16-byte LDS reads.
+template <int R, int K, bool VEC, bool LOCAL, int NT> __global__ void __launch_bounds__(NT) ssd_scan_lds_kernel(ScanArgs a, int rowpad) {
+  constexpr int TC = 8;  // rows per stage; a thread stages columns tid and tid + nthr of every row (16 registers)
+  extern __shared__ __attribute__((aligned(16))) float sm[];  // [2][TC][rowpad]: B [N] | C [N] | x [P] | dt | decay
+  constexpr int PT = 64 / R;
+  const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, r = lane % R, p = wave * PT + lane / R;
+  const int h = blockIdx.y, z = blockIdx.z;
+  const int s = a.seg_entry[z], r0 = a.seg_row0[z], len = a.seg_len[z];
+  const bool first = z == a.ent_seg0[s], last = z == a.ent_seg0[s + 1] - 1;
+  if (len <= 0 || (LOCAL && last)) return;
+  const bool live = p < a.P;
+  const int pc = live ? p : a.P - 1;
+  const int g = h / (a.heads / a.G), inner = a.heads * a.P, N = a.N, P = a.P;
+  int nk = N - r * K;
+  nk = nk < 0 ? 0 : (nk > K ? K : nk);
+  const size_t np = (size_t)N * P;
+  float *st = a.state + ((size_t)a.seq_slot[s] * a.heads + h) * np;
+  const float *init = LOCAL ? nullptr : (first ? (a.seq_pos0[s] > 0 ? st : nullptr) : a.carry + ((size_t)(z - 1) * a.heads + h) * np);
+  float S[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) S[k] = (k < nk && init) ? init[(size_t)(r * K + k) * P + pc] : 0.f;
+  const float Dh = a.D[h];
+  const int bcol = inner + g * N, ccol = inner + a.G * N + g * N, per = TC * rowpad, rowlen = 2 * N + P + 2;
+  float stg[16], prod = 1.0f;
+  auto fetch = [&](int c0) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int tok = q >> 1, j = tid + (q & 1) * nthr, i = c0 + tok;
+      float v = 0.f;
+      if (i < len && j < rowlen) {
+        const int row = r0 + i;
+        const float *xr = a.xbc + (size_t)row * a.C;
+        if (j < N) v = xr[bcol + j];
+        else if (j < 2 * N) v = xr[ccol + j - N];
+        else if (j < 2 * N + P) v = xr[h * P + j - 2 * N];
+        else v = a.steps[2 * ((size_t)row * a.heads + h) + (j - 2 * N - P)];
+      }
+      stg[q] = v;
+    }
+  };
+  auto put = [&](float *buf) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const int j = tid + (q & 1) * nthr;
+      if (j < rowpad) buf[(q >> 1) * rowpad + j] = stg[q];
+    }
+  };
+  fetch(0);
+  put(sm);
+  __syncthreads();
+  int flip = 0;
+  for (int c0 = 0; c0 < len; c0 += TC, flip ^= 1) {
+    const float *cur = sm + flip * per;
+    const bool more = c0 + TC < len;
+    if (more) fetch(c0 + TC);
+    const int cnt = len - c0 < TC ? len - c0 : TC;
+    for (int j = 0; j < cnt; ++j) {
+      const float *row = cur + j * rowpad;
+      const float dt = row[2 * N + P], dec = row[2 * N + P + 1], xv = row[2 * N + pc];
+      const float dx = dt * xv;
+      float part = 0.f;
+      if (VEC) {
+#pragma unroll
+        for (int k = 0; k < K; k += 4) {
+          const int kk = r * K + (k < nk ? k : 0);
+          const float4 b4 = *(const float4 *)(row + (nk ? kk : 0)), c4 = *(const float4 *)(row + N + (nk ? kk : 0));
+          const bool on = k < nk;
+          const float bb[4] = {on ? b4.x : 0.f, on ? b4.y : 0.f, on ? b4.z : 0.f, on ? b4.w : 0.f}, cc[4] = {on ? c4.x : 0.f, on ? c4.y : 0.f, on ? c4.z : 0.f, on ? c4.w : 0.f};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            S[k + q] = fmaf(dec, S[k + q], dx * bb[q]);
+            if (!LOCAL) part = fmaf(S[k + q], cc[q], part);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          const int kk = k < nk ? r * K + k : 0;
+          const float bv = k < nk ? row[kk] : 0.f, cv = k < nk ? row[N + kk] : 0.f;
+          S[k] = fmaf(dec, S[k], dx * bv);
+          if (!LOCAL) part = fmaf(S[k], cv, part);
+        }
+      }
+      if (LOCAL) prod *= dec;
+      else {
+#pragma unroll
+        for (int m = 1; m < R; m <<= 1) part += __shfl_xor(part, m, 64);
+        if (r == 0 && live) a.out[(size_t)(r0 + c0 + j) * inner + h * P + p] = fmaf(Dh, xv, part);
+      }
+    }
+    if (more) put(sm + (flip ^ 1) * per);
+    __syncthreads();
+  }
+  if (LOCAL) {
+    if (tid == 0) a.decay[(size_t)z * a.heads + h] = prod;
+    st = a.carry + ((size_t)z * a.heads + h) * np;
+  }
+  if (live && (LOCAL || last))
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      if (k < nk) st[(size_t)(r * K + k) * P + p] = S[k];
+}
+
 // ---------------------------------------------------------------------------------- query / key norm over the whole projection, partial interleaved rotary, K / V page write
 struct QkArgs {
   const float *qkv;   // [rows, ld]: q [H * D] | k [G * D] | v [G * Dv]
@@ -632,10 +737,23 @@ extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *d
   if (!single) hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
   const bool split = segments > entries;
 #define MRS_SCAN_(R, K, V, DP, L) hipLaunchKernelGGL((ssd_scan_kernel<R, K, V, DP, L>), dim3((P + 64 / R - 1) / (64 / R), heads, segments), dim3(64), 0, S_(stream), a)
+#define MRS_SCAN_LDS_(R, K, V, L) do { if (nw <= 4) hipLaunchKernelGGL((ssd_scan_lds_kernel<R, K, V, L, 256>), dim3(1, heads, segments), dim3(64 * nw), lds_bytes, S_(stream), a, rowpad); \
+                                       else hipLaunchKernelGGL((ssd_scan_lds_kernel<R, K, V, L, 1024>), dim3(1, heads, segments), dim3(64 * nw), lds_bytes, S_(stream), a, rowpad); } while (0)
+  // portions: the LDS-staged kernel when one workgroup can hold a head's P (<= 16 waves) and two columns per thread cover a staged row
+  int nw = 0;
+  const int rowpad = (2 * N + P + 2 + 3) & ~3;
+  const size_t lds_bytes = (size_t)2 * 8 * rowpad * 4;
+  auto plan_lds = [&](int R_) {
+    nw = (P + 64 / R_ - 1) / (64 / R_);
+    if (single || nw > 16 || rowpad > 2 * 64 * nw || lds_bytes > 65536) nw = 0;
+  };
 #define MRS_SCAN(R, K, DP) do { \
-    if (split) { if (vec) MRS_SCAN_(R, K, true, DP, true); else MRS_SCAN_(R, K, false, DP, true); \
+    plan_lds(R); \
+    if (split) { if (nw) { if (vec) MRS_SCAN_LDS_(R, K, true, true); else MRS_SCAN_LDS_(R, K, false, true); } \
+                 else { if (vec) MRS_SCAN_(R, K, true, DP, true); else MRS_SCAN_(R, K, false, DP, true); } \
                  hipLaunchKernelGGL(ssd_carry_kernel, dim3((N * P + 255) / 256, heads, entries), dim3(256), 0, S_(stream), a); } \
     if (single) { if (vec) MRS_SCAN_(R, K, true, 1, false); else MRS_SCAN_(R, K, false, 1, false); } \
+    else if (nw) { if (vec) MRS_SCAN_LDS_(R, K, true, false); else MRS_SCAN_LDS_(R, K, false, false); } \
     else { if (vec) MRS_SCAN_(R, K, true, DP, false); else MRS_SCAN_(R, K, false, DP, false); } } while (0)
   if (N <= 16) MRS_SCAN(2, 8, 8);
   else if (N <= 64) MRS_SCAN(4, 16, 6);
@@ -643,6 +761,7 @@ extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *d
   else if (N <= 256) MRS_SCAN(8, 32, 4);
   else if (N <= 512) MRS_SCAN(16, 32, 4);
   else return fail("mrs_hyb_ssd_scan: state size above 512");
+#undef MRS_SCAN_LDS_
 #undef MRS_SCAN
 #undef MRS_SCAN_
   return ok_or("mrs_hyb_ssd_scan");
