@@ -560,6 +560,118 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
   }
 }
 
+// Portions: NQ consecutive queries of one entry (a tile of a segment) per wave.  A key row is loaded once and scored against all NQ queries (their vectors sit in LDS),
+// a value pair is loaded once and added into NQ accumulators: 1 / NQ of the single-query kernel's loads for the same arithmetic.  Every query keeps its own running
+// maximum / sum and its own visibility test (position i sees key j <= i with i - j < window or j < keep_first); the key range of the tile is the union of its queries' ranges.
+template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_window_attn_tile_kernel(AttnArgs a, const int *__restrict__ seg_entry, const int *__restrict__ seg_row0,
+                                                                                                        const int *__restrict__ seg_len) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // q [NQ][Dp] | p [64][NQ] | key row index [64]
+  const int z = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
+  const int t0 = seg_row0[z] + blockIdx.x * NQ;
+  int nq = seg_row0[z] + seg_len[z] - t0;
+  if (nq <= 0) return;
+  nq = nq > NQ ? NQ : nq;
+  const int Dp = (a.D + 3) & ~3;
+  float *qs = lds, *ps = lds + NQ * Dp;
+  long long *rowbase = (long long *)(ps + 64 * NQ);
+  const int s = seg_entry[z], i0 = a.tok_pos[t0], g = h / (a.H / a.G);
+  for (int e = lane; e < NQ * Dp; e += 64) {
+    const int q = e / Dp, d = e - q * Dp;
+    qs[e] = (q < nq && d < a.D) ? to_f<T>(((const T *)a.q)[((size_t)(t0 + q) * a.H + h) * a.D + d]) : 0.f;
+  }
+  const int *bt = a.block_tables + (size_t)s * a.max_blocks;
+  int w_lo = a.window > 0 ? i0 - a.window + 1 : 0;
+  if (w_lo < 0) w_lo = 0;
+  int n1 = a.keep_first < w_lo ? a.keep_first : w_lo;
+  if (n1 < 0) n1 = 0;
+  const int total = n1 + (i0 + nq - 1 - w_lo + 1);
+  float m[NQ], l[NQ], o[NQ][DVC][2];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    m[q] = -FLT_MAX; l[q] = 0.f;
+#pragma unroll
+    for (int c = 0; c < DVC; ++c) o[q][c][0] = o[q][c][1] = 0.f;
+  }
+  MRS_WAVE_SYNC();
+  for (int v0 = 0; v0 < total; v0 += 64) {
+    const int vi = v0 + lane;
+    int key = -1;
+    long long base = -1;
+    float sc[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) sc[q] = 0.f;
+    if (vi < total) {
+      key = vi < n1 ? vi : w_lo + (vi - n1);
+      base = ((long long)bt[key / a.block_size] * a.G + g) * a.block_size + key % a.block_size;
+      const T *kr = (const T *)a.k_cache + (size_t)base * a.D;
+      for (int d = 0; d < a.D; d += 8) {
+        float kv[8];
+        Ld<T>::v8(kr + d, kv);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          const float4 qa = *(const float4 *)(qs + q * Dp + d), qb = *(const float4 *)(qs + q * Dp + d + 4);
+          float acc = sc[q];
+          acc = fmaf(qa.x, kv[0], acc); acc = fmaf(qa.y, kv[1], acc); acc = fmaf(qa.z, kv[2], acc); acc = fmaf(qa.w, kv[3], acc);
+          acc = fmaf(qb.x, kv[4], acc); acc = fmaf(qb.y, kv[5], acc); acc = fmaf(qb.z, kv[6], acc); acc = fmaf(qb.w, kv[7], acc);
+          sc[q] = acc;
+        }
+      }
+    }
+    MRS_WAVE_SYNC();  // the previous pass has read p and the row indices
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int iq = i0 + q;
+      const bool vis = key >= 0 && q < nq && key <= iq && (a.window <= 0 || iq - key < a.window || key < a.keep_first);
+      const float sv = vis ? sc[q] * a.scale : -FLT_MAX;
+      const float mn = fmaxf(m[q], wave_max(sv));
+      const float alpha = expf(m[q] - mn);
+      const float pq = vis ? expf(sv - mn) : 0.f;
+      l[q] = l[q] * alpha + wave_sum(pq);
+      m[q] = mn;
+#pragma unroll
+      for (int c = 0; c < DVC; ++c) { o[q][c][0] *= alpha; o[q][c][1] *= alpha; }
+      ps[lane * NQ + q] = pq;
+    }
+    rowbase[lane] = base;
+    MRS_WAVE_SYNC();
+    const int cnt = total - v0 < 64 ? total - v0 : 64;
+#pragma unroll
+    for (int c = 0; c < DVC; ++c) {
+      const int d = 128 * c + 2 * lane;
+      if (d < a.Dv) {
+        const T *vb = (const T *)a.v_cache + d;
+#pragma unroll 2
+        for (int j = 0; j < cnt; ++j) {
+          float x, y;
+          Ld<T>::v2(vb + (size_t)rowbase[j] * a.Dv, x, y);
+          float pj[NQ];
+#pragma unroll
+          for (int q4 = 0; q4 < NQ; q4 += 4) {
+            const float4 p4 = *(const float4 *)(ps + j * NQ + q4);
+            pj[q4] = p4.x; pj[q4 + 1] = p4.y; pj[q4 + 2] = p4.z; pj[q4 + 3] = p4.w;
+          }
+#pragma unroll
+          for (int q = 0; q < NQ; ++q) {
+            o[q][c][0] = fmaf(pj[q], x, o[q][c][0]);
+            o[q][c][1] = fmaf(pj[q], y, o[q][c][1]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    if (q >= nq) break;
+    const float inv = 1.0f / l[q];
+    T *out = (T *)a.out + ((size_t)(t0 + q) * a.H + h) * a.Dv;
+#pragma unroll
+    for (int c = 0; c < DVC; ++c) {
+      const int d = 128 * c + 2 * lane;
+      if (d < a.Dv) { out[d] = from_f<T>(o[q][c][0] * inv); out[d + 1] = from_f<T>(o[q][c][1] * inv); }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------- mixture of experts: routing, dispatch, gather, GLU, combine
 // Router: one workgroup per row.  logits z_e = w_e . h in f32 (a wave per expert, lanes over the width, butterfly sum), score = sigmoid(z); the `top` largest (ties: the
 // lower index), weights = the scores, un-renormalised; row E of the weight (when has_gate) is the shared expert's gate: gate[t] = sigmoid(w_E . h).
@@ -779,17 +891,33 @@ extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float 
   return ok_or("mrs_hyb_qk_norm_rope_cache");
 }
 
+/* seg_entry / seg_row0 / seg_len [segments] (nullable): the batch's segment table (rows of one entry in pieces); with it, batches that bring portions run the
+ * query-tiled kernel */
 extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
-                                         int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype, void *stream) {
+                                         int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
+                                         const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, void *stream) {
   if (rows <= 0) return 0;
   if (Dv > 256 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 256 / heads % kv_heads");
   AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale};
+  const bool vec = D % 8 == 0 && Dv % 2 == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 8) == 0;
+  const int c = (Dv + 127) / 128;
+  if (vec && seg_entry && segments > 0 && rows > segments && segments <= 65535 && seg_rows > 0) {
+    constexpr int NQ = 8;
+    const size_t lds = (size_t)(NQ * ((D + 3) & ~3) + 64 * NQ) * 4 + 64 * 8;
+    if (lds <= 65536) {
+      dim3 grid((seg_rows + NQ - 1) / NQ, H, segments);
+#define MRS_ATTN_T(T, C) hipLaunchKernelGGL((paged_window_attn_tile_kernel<T, C, NQ>), grid, dim3(64), lds, S_(stream), a, seg_entry, seg_row0, seg_len)
+      if (dtype == 1) { if (c <= 1) MRS_ATTN_T(mrs::bf16_t, 1); else MRS_ATTN_T(mrs::bf16_t, 2); }
+      else if (dtype == 2) { if (c <= 1) MRS_ATTN_T(float, 1); else MRS_ATTN_T(float, 2); }
+      else return fail("mrs_hyb_paged_window_attn: dtype");
+#undef MRS_ATTN_T
+      return ok_or("mrs_hyb_paged_window_attn");
+    }
+  }
   const size_t lds = (size_t)(((D + 3) & ~3) + 64) * 4 + 64 * 8;
   dim3 grid(rows, H);
-  const bool vec = D % 8 == 0 && Dv % 2 == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 8) == 0;
 #define MRS_ATTN(T, C) do { if (vec) hipLaunchKernelGGL((paged_window_attn_kernel<T, C, true>), grid, dim3(64), lds, S_(stream), a); \
                             else hipLaunchKernelGGL((paged_window_attn_kernel<T, C, false>), grid, dim3(64), lds, S_(stream), a); } while (0)
-  const int c = (Dv + 127) / 128;
   if (dtype == 1) { if (c <= 1) MRS_ATTN(mrs::bf16_t, 1); else MRS_ATTN(mrs::bf16_t, 2); }
   else if (dtype == 2) { if (c <= 1) MRS_ATTN(float, 1); else MRS_ATTN(float, 2); }
   else return fail("mrs_hyb_paged_window_attn: dtype");

@@ -34,7 +34,7 @@ _SIGS = {
     "mrs_hyb_conv_silu": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "mrs_hyb_ssd_scan": [_vp] * 16 + [_i] * 10 + [_vp],
     "mrs_hyb_qk_norm_rope_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
-    "mrs_hyb_paged_window_attn": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp],
+    "mrs_hyb_paged_window_attn": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp, _vp, _vp, _i, _i, _vp],
     "mrs_hyb_route_sigmoid_topk": [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp],
     "mrs_hyb_moe_dispatch": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp],
     "mrs_hyb_moe_gather": [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp],
@@ -330,7 +330,7 @@ class WindowAttention(_Module):
               s.heads, s.kv_heads, s.dim, s.vdim, s.rotary.dims if s.rotary else 0, m.block_size, m.spec.eps, m.dt)
         o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
         _call("mrs_hyb_paged_window_attn", q, self.k_cache, self.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size,
-              b.max_blocks, s.window, s.keep_first, s.scale, m.dt)
+              b.max_blocks, s.window, s.keep_first, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
         m.linear(o, self.w_o, out=x, accumulate=True)
 
 

@@ -367,7 +367,8 @@ def test_planted_keys_at_every_edge(dev, dtype):
             qq = torch.zeros(n, H * D, dtype=td, device=dev)
             qq[n - 1] = q.reshape(-1).to(dev, td)
             out = torch.empty(n, H * Dv, dtype=td, device=dev)
-            _call("mrs_hyb_paged_window_attn", qq, att.k_cache, att.v_cache, b.block_tables, b.tok_seq, b.tok_pos, out, n, H, G, D, Dv, bs, b.max_blocks, size, keep, 1.0, m.dt)
+            _call("mrs_hyb_paged_window_attn", qq, att.k_cache, att.v_cache, b.block_tables, b.tok_seq, b.tok_pos, out, n, H, G, D, Dv, bs, b.max_blocks, size, keep, 1.0, m.dt,
+                  b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
             got = out[n - 1].double().cpu().view(H, Dv)
             assert rel(got, want[0]) < (1e-5 if dtype == "float32" else 1e-2), (i, j, rows, seen)
     sv.end(1)
