@@ -15,14 +15,14 @@ import json
 import sys
 
 
-def make_engine(model, max_tokens: int, max_seqs: int, sampler=None, max_batched_tokens: int = 2048):
+def make_engine(model, max_tokens: int, max_seqs: int, sampler=None, max_batched_tokens: int = 2048, use_graphs: bool = True):
     """Scheduler + engine around a loaded model with a ragged step function (hybrid.HybridDecoder): pages for `max_tokens` live tokens, `max_seqs` state slots."""
     from .hybrid import HybridCache
     from .scheduler import PagedAttentionScheduler, PagedEngine, SchedulerConfig
     cache = HybridCache(model)
     sched = PagedAttentionScheduler(SchedulerConfig(max_num_seqs=max_seqs, max_num_batched_tokens=max_batched_tokens, uniform_prompt_batches=False), cache.kv,
                                     prefix_caching=False, state_pool=cache.slots if model.has_recurrent_state else None)
-    eng = PagedEngine(model, sched, sampler=sampler)
+    eng = PagedEngine(model, sched, sampler=sampler, use_graphs=use_graphs)
     eng.cache = cache
     return eng
 

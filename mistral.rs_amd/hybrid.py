@@ -45,6 +45,7 @@ _SIGS = {
     "mrs_hyb_gemv": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp],
 }
 _fns: dict = {}
+_step_stream: Optional[int] = None   # the stream handle of the step in progress (looked up once per forward_batch, not once per launch)
 
 
 def _call(name: str, *args) -> None:
@@ -53,7 +54,7 @@ def _call(name: str, *args) -> None:
     if fn is None:
         fn = _fns[name] = _lib.sym("hybrid", name, _SIGS[name], C.c_int)
     conv = [a.data_ptr() if isinstance(a, torch.Tensor) else a for a in args]
-    if fn(*conv, torch.cuda.current_stream().cuda_stream) != 0:
+    if fn(*conv, _step_stream if _step_stream is not None else torch.cuda.current_stream().cuda_stream) != 0:
         err = _lib.sym("hybrid", "mrs_hyb_gemm_last_error" if "gem" in name else "mrs_hyb_last_error", [], C.c_char_p)()
         raise ValueError((err or b"").decode() or name)
 
@@ -495,6 +496,14 @@ class HybridDecoder:
     # ---- the step
     def forward_batch(self, b: RaggedBatch) -> torch.Tensor:
         """Runs the batch's rows from the cache and state that earlier steps left; returns f32 logits [len(want), vocab] in the order of `want`."""
+        global _step_stream
+        _step_stream = torch.cuda.current_stream().cuda_stream
+        try:
+            return self._forward_batch(b)
+        finally:
+            _step_stream = None
+
+    def _forward_batch(self, b: RaggedBatch) -> torch.Tensor:
         sp = self.spec
         T = b.rows
         if T == 0:

@@ -312,8 +312,10 @@ class PagedEngine:
     `prompt_chunk_size` tokens through the same kernels (so a preempted and recomputed sequence reproduces its logits bit for bit), block tables and slot
     mappings from the KV cache manager (pipeline/inputs_processor.rs:900-922)."""
 
-    def __init__(self, model, scheduler: PagedAttentionScheduler, sampler=None):
+    def __init__(self, model, scheduler: PagedAttentionScheduler, sampler=None, use_graphs: bool = False):
         self.m, self.s = model, scheduler
+        self.use_graphs = use_graphs   # ragged models: completion passes replay a HIP graph of the decode step (one per batch size, captured on first use)
+        self._graphs: dict = {}
         self.ragged = hasattr(model, "forward_batch")  # a ragged step function: unequal prompt portions and single tokens in one call
         self.cfg = None if self.ragged else model.cfg
         self.max_context_len = scheduler.kv.num_gpu_blocks() * scheduler.block_size if self.ragged else model.cfg.max_context_len
@@ -350,7 +352,13 @@ class PagedEngine:
             ends.append((seq, b))
         if not entries:
             return
-        logits = self.m.forward_batch(RaggedBatch.build(entries, self.s.block_size, self.m.device))
+        if out.kind == "completion" and self.use_graphs and all(len(e["tokens"]) == 1 for e in entries):
+            g = self._graphs.get(len(entries))
+            if g is None:  # the table width covers the longest sequence the pool can hold
+                g = self._graphs[len(entries)] = self.m.capture_decode(len(entries), self.s.kv.num_gpu_blocks())
+            logits = g.replay(entries)
+        else:
+            logits = self.m.forward_batch(RaggedBatch.build(entries, self.s.block_size, self.m.device))
         row = 0
         for seq, b in ends:
             seq.num_computed_tokens = b

@@ -475,7 +475,8 @@ def test_sizes_that_coincide_or_equal_one(dev):
 
 
 @pytest.mark.gpu
-def test_greedy_generation_through_scheduler_and_engine(dev):
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+def test_greedy_generation_through_scheduler_and_engine(dev, graphs):
     """the package's own entry point: scheduler (pages + state slots), engine, sampler (top-1 kernels); five prompts through three slots, against greedy decoding of the restatement"""
     from mistralrs_amd.cli import make_engine
     from mistralrs_amd.hybrid import HybridDecoder, gekilix_spec
@@ -486,7 +487,7 @@ def test_greedy_generation_through_scheduler_and_engine(dev):
     m = HybridDecoder(gekilix_spec(cfg), dev, "float32", num_blocks=12, block_size=32, state_slots=3)
     m.load_weights(w.__getitem__)
     core = os.path.exists(_lib.path("core"))
-    eng = make_engine(m, 12 * 32, 3, sampler=SequenceSampler(cfg["vocab"], dev, top_k=1) if core else None, max_batched_tokens=48)
+    eng = make_engine(m, 12 * 32, 3, sampler=SequenceSampler(cfg["vocab"], dev, top_k=1) if core else None, max_batched_tokens=48, use_graphs=graphs)
     prompts = [toks(n, cfg["vocab"], 20 + n) for n in (5, 40, 1, 23, 60)]
     seqs = [Sequence(id=i + 1, tokens=list(p), max_new_tokens=6) for i, p in enumerate(prompts)]
     for s in seqs:
@@ -503,6 +504,7 @@ def test_greedy_generation_through_scheduler_and_engine(dev):
             ref.append(int(lg.argmax()))
         assert s.error is None and s.generated[:len(ref) - len(p)] == ref[len(p):], (s.id, s.generated, ref[len(p):])
     assert eng.s.state_pool.num_free_slots() == 3 and eng.steps["prompt"] >= 2 and eng.steps["completion"] >= 6
+    assert bool(eng._graphs) == graphs
 
 
 @pytest.mark.gpu
@@ -530,3 +532,55 @@ def test_captured_decode_steps_equal_eager_steps(dev):
         got = g.replay(entries).double().cpu()
         assert rel(got, want) < 1e-6, f"replay {i}"
         torch.cuda.synchronize()
+
+
+@pytest.mark.gpu
+def test_checkpoint_folder_through_registry_command_line_and_trace_replay(dev, tmp_path, monkeypatch, capsys):
+    """config.json + model.safetensors on disk -> registry -> `generate` (scheduler, engine, sampler) and `trace` (steps from standard input, logits to files, pages and
+    slots given back and reused) -- both against the restatement"""
+    import io
+    from safetensors.torch import save_file
+    from mistralrs_amd import cli, registry, trace
+    cfg = config([mamba_layer(top=1), attn_layer(top=2, size=10, keep=1)])
+    w = weights(cfg, 9)
+    folder = tmp_path / "model"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in w.items()}, str(folder / "model.safetensors"))
+    assert registry.architecture_of(str(folder)) == "Gekilix"
+    wd = f64(w)
+    # ---- trace replay: three requests through two state slots and a pool of 128 tokens, portions beside single tokens, an empty `want`
+    reqs = {"a": toks(45, cfg["vocab"], 51), "b": toks(20, cfg["vocab"], 52), "c": toks(33, cfg["vocab"], 53)}
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": reqs["a"][:30], "want": [0, 29]}, {"id": "b", "tokens": reqs["b"][:19], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": reqs["a"][30:31], "want": [0]}, {"id": "b", "tokens": reqs["b"][19:], "want": [0]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "c", "tokens": reqs["c"][:2], "want": [1]}, {"id": "a", "tokens": reqs["a"][31:], "want": [13]}], "end": ["a"]},
+             {"step": 3, "entries": [{"id": "c", "tokens": reqs["c"][2:], "want": [0, 30]}], "end": ["c"]}]
+    out = tmp_path / "out"
+    monkeypatch.setattr("sys.stdin", io.StringIO("\n".join(json.dumps(s) for s in steps) + "\n"))
+    assert trace.main(["--model", str(folder), "--dtype", "float32", "--out", str(out), "--max-tokens", "128", "--state-slots", "2"]) == 0
+    printed = capsys.readouterr().out.split("\n")
+    assert [l for l in printed if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    full = {r: O.forward(cfg, wd, t) for r, t in reqs.items()}
+    want = {0: [full["a"][0], full["a"][29]], 1: [full["a"][30], full["b"][19]], 2: [full["c"][1], full["a"][44]], 3: [full["c"][2], full["c"][32]]}
+    for n, rows in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"]).astype(np.float64))
+        assert rel(got, torch.stack(rows)) < 3e-5, f"step {n}"
+    # ---- generate: greedy, two prompts
+    prompts = [toks(12, cfg["vocab"], 61), toks(3, cfg["vocab"], 62)]
+    args = ["generate", "--model", str(folder), "--dtype", "float32", "--max-new-tokens", "4", "--max-tokens", "256", "--max-seqs", "2"]
+    for p in prompts:
+        args += ["--prompt-ids", ",".join(map(str, p))]
+    if not os.path.exists(_lib.path("core")):
+        pytest.skip("the sampler's library is not built")
+    assert cli.main(args) == 0
+    lines = [json.loads(l) for l in capsys.readouterr().out.split("\n") if l.startswith("{")]
+    assert len(lines) == 2
+    for p, line in zip(prompts, lines):
+        ref = list(p)
+        for _ in range(4):
+            lg = O.forward(cfg, wd, ref)[-1]
+            t2 = torch.topk(lg, 2).values
+            if float(t2[0] - t2[1]) < 1e-3:
+                break
+            ref.append(int(lg.argmax()))
+        assert line["error"] is None and line["tokens"][:len(ref) - len(p)] == ref[len(p):]
