@@ -27,7 +27,7 @@ def rms_unit(x, eps):
 
 
 def norm_one_plus(x, w, eps):
-    """Layer norm of the family: unit RMS, then (1 + w) (the weight is stored around zero)."""
+    """Layer norm of the family: unit RMS, then (1 + w) (weights are kept as offsets from one)."""
     return rms_unit(x, eps) * (1.0 + w)
 
 
