@@ -82,7 +82,7 @@ class RaggedBatch:
     seg_len: Optional[torch.Tensor] = None     # i32 [segments]
     ent_seg0: Optional[torch.Tensor] = None    # i32 [entries + 1]  first segment of every entry, then the total
 
-    SEGMENT = 128
+    SEGMENT = int(os.environ.get("MRS_HYB_SEGMENT", "64"))   # rows per segment
 
     @staticmethod
     def build(entries: Sequence[dict], block_size: int, device) -> "RaggedBatch":
