@@ -584,3 +584,23 @@ def test_checkpoint_folder_through_registry_command_line_and_trace_replay(dev, t
                 break
             ref.append(int(lg.argmax()))
         assert line["error"] is None and line["tokens"][:len(ref) - len(p)] == ref[len(p):]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,bar", [("float32", 3e-5), ("bfloat16", 5e-2)])
+def test_sizes_off_every_vector_width(dev, dtype, bar):
+    """a width of 30, an odd value size, a key size of 6, expert sizes of 10 and 7, a state size of 9: nothing is a multiple of 4 or 8, so every kernel runs its element-wise
+    path -- whole prompt, portions and single steps (whose products build their operands in the load)"""
+    layers = [mamba_layer(heads=3, vdim=5, state=9, groups=1, conv=3, norm_groups=3, experts=4, top=2, ff=10, shared=7),
+              attn_layer(heads=4, kv_heads=2, dim=6, vdim=5, size=11, keep=2, rot=4, experts=3, top=1, ff=7, shared=0),
+              attn_layer(heads=2, kv_heads=1, dim=8, vdim=3, size=200, keep=0, rot=8, scaling=False, mlp=False)]
+    cfg = config(layers, vocab=51, width=30, eps=1e-6)
+    w = weights(cfg, 12)
+    t = toks(80, 51, 9)
+    want = O.forward(cfg, f64(w), t)
+    sv = Served(cfg, w, dev, dtype)
+    assert close(sv.step([(1, t)])[0], want, bar)
+    got = torch.cat([sv.step([(2, t[:70])])[0]] + [sv.step([(2, [x])])[0] for x in t[70:]])
+    assert close(got, want, bar)
+    mixed = sv.step([(3, t[:9]), (4, t[:1])])
+    assert close(mixed[0], want[:9], bar) and close(mixed[1], want[:1], bar)
