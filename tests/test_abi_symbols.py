@@ -13,6 +13,7 @@ HEADER_LIB = {
     "mistralrs_paged_attn.h": "libmistralrspagedattention.so",
     "mistralrs_core.h": "libmistralrscuda.so",
     "mrs_hip_ext.h": "libmrs_hip_ext.so",
+    "mrs_hybrid.h": "libmrs_hybrid.so",
 }
 
 
