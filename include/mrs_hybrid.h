@@ -27,10 +27,20 @@ int mrs_hyb_moe_gather(const float *h32, const int *sorted_route, const float *w
 int mrs_hyb_glu_silu(const float *gu, void *out, int rows, int ff, int dtype, void *stream);
 int mrs_hyb_moe_combine(float *x, const float *d, const int *route_pos, int top, const float *shared, const float *gate, int rows, int W, void *stream);
 int mrs_hyb_gather_rows(const float *x, const int *idx, float *out, int n, int W, void *stream);
+int mrs_hyb_route_softmax_topk(const float *h, const float *wr, int rows, int W, int E, int top, float scale, int *ids, float *wts, void *stream);
+int mrs_hyb_moe_combine_weighted(float *out, const float *d, const int *route_pos, const float *wts, int top, const float *shared, int rows, int W, int accumulate, void *stream);
+int mrs_hyb_glu_clamped(const float *gu, void *out, int rows, int ff, float limit, float alpha, int dtype, void *stream);
+int mrs_hyb_bias_xielu(const float *u, int ldu, const float *bias, void *out, int rows, int ff, float ap, float an, int dtype, void *stream);
+int mrs_hyb_layernorm(const float *x, int ldx, const float *in_bias, const float *w, const float *b, void *out, float *out32, float *resid, int ldr, int rows, int width, float eps, int dtype, void *stream);
+int mrs_hyb_qkv_bias_temp_cache(const float *qkv, int ld, const float *qb, const float *kb, const float *vb, const int *tok_pos, const long long *slot_mapping, void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int block_size, float temp_coef, int temp_every, int dtype, void *stream);
+/* ---- hyb_attn_talk.hip */
+const char *mrs_hyb_talk_last_error();
+int mrs_hyb_paged_talk_sigmoid_attn(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_pos, const float *talk, const float *pb, const float *slopes, const float *gate, int ldg, void *out, int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, float scale, int dtype, const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, void *stream);
 /* ---- hyb_gemm.hip */
 const char *mrs_hyb_gemm_last_error();
 int mrs_hyb_gemm(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate, const int *bounds, int groups, long long wstride, int max_rows, void *stream);
 int mrs_hyb_gemv(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate, const int *row_group, long long wstride, int in_mode, const int *src_row, const float *src_scale, int src_div, void *stream);
+int mrs_hyb_gemv_act(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate, const int *row_group, long long wstride, int in_mode, const int *src_row, const float *src_scale, int src_div, const float *in_bias, float p0, float p1, void *stream);
 void *mrs_state_pool_create(size_t num_slots);
 void mrs_state_pool_destroy(void *h);
 size_t mrs_state_pool_capacity(void *h);

@@ -257,8 +257,11 @@ __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
 // The activation operand of a row kernel can be produced on the fly (decode steps: one launch less per use):
 //   IN_PLAIN   A [M, K] in T
 //   IN_GLU     A = f32 [M, 2 K] = gate | up of the previous product: x_k = round_T(silu(gate_k) * up_k)
-//   IN_SCALED  A = f32 [rows, K] normed rows: row m reads source row src_row[m] / src_div times src_scale[src_row[m]], rounded to T (expert-sorted routed inputs)
-enum { IN_PLAIN = 0, IN_GLU = 1, IN_SCALED = 2 };
+//   IN_SCALED  A = f32 [rows, K] normed rows: row m reads source row src_row[m] / src_div times src_scale[src_row[m]] (1 without scales), rounded to T (expert-sorted
+//              routed inputs)
+//   IN_GLU_CLAMP  A = f32 [M, 2 K] = gate | up: g = min(gate, p0), u = clamp(up, -p0, p0): x_k = round_T(g sigmoid(p1 g) (u + 1))
+//   IN_BIAS_XIELU A = f32 [M, K]: z = A + in_bias: x_k = round_T(z > 0 ? p0 z^2 + z / 2 : p1 (e^z - 1 - z) + z / 2)
+enum { IN_PLAIN = 0, IN_GLU = 1, IN_SCALED = 2, IN_GLU_CLAMP = 3, IN_BIAS_XIELU = 4 };
 struct GemvArgs {
   const void *A;
   const void *W;
@@ -271,6 +274,8 @@ struct GemvArgs {
   const int *src_row;        // IN_SCALED
   const float *src_scale;
   int src_div;
+  const float *in_bias;      // IN_BIAS_XIELU
+  float p0, p1;              // IN_GLU_CLAMP: limit, sigmoid factor; IN_BIAS_XIELU: the two coefficients
 };
 
 template <class T> struct Vec8;
@@ -296,14 +301,21 @@ template <> struct Vec8<float> {
   static __device__ __forceinline__ void load_nt(const float *p, float *o) { load(p, o); }
 };
 __device__ __forceinline__ float silu_in(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float glu_clamp_in(float gv, float uv, float limit, float alpha) {
+  const float g = fminf(gv, limit), u = fminf(fmaxf(uv, -limit), limit);
+  return g * (1.0f / (1.0f + expf(-(alpha * g)))) * (u + 1.0f);
+}
+__device__ __forceinline__ float xielu_in(float z, float ap, float an) { return z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(an, expm1f(z) - z, 0.5f * z); }
 
 // one activation value (element path) / eight (vector path) of row m at column k, as the product sees it
 template <class T, int IN> __device__ __forceinline__ float act1(const GemvArgs &a, int m, int k) {
   if (IN == IN_PLAIN) return to_f<T>(((const T *)a.A)[(size_t)m * a.lda + k]);
   const float *A = (const float *)a.A;
   if (IN == IN_GLU) return round_to<T>(silu_in(A[(size_t)m * a.lda + k]) * A[(size_t)m * a.lda + a.K + k]);
+  if (IN == IN_GLU_CLAMP) return round_to<T>(glu_clamp_in(A[(size_t)m * a.lda + k], A[(size_t)m * a.lda + a.K + k], a.p0, a.p1));
+  if (IN == IN_BIAS_XIELU) return round_to<T>(xielu_in(A[(size_t)m * a.lda + k] + (a.in_bias ? a.in_bias[k] : 0.f), a.p0, a.p1));
   const int r = a.src_row[m];
-  return round_to<T>(a.src_scale[r] * A[(size_t)(r / a.src_div) * a.lda + k]);
+  return round_to<T>((a.src_scale ? a.src_scale[r] : 1.0f) * A[(size_t)(r / a.src_div) * a.lda + k]);
 }
 template <class T, int IN> __device__ __forceinline__ void act8(const GemvArgs &a, int m, int k, float *x) {
   if (IN == IN_PLAIN) { Vec8<T>::load((const T *)a.A + (size_t)m * a.lda + k, x); return; }
@@ -316,8 +328,24 @@ template <class T, int IN> __device__ __forceinline__ void act8(const GemvArgs &
     for (int j = 0; j < 8; ++j) x[j] = round_to<T>(silu_in(g[j]) * u[j]);
     return;
   }
+  if (IN == IN_GLU_CLAMP) {
+    float g[8], u[8];
+    Vec8<float>::load(A + (size_t)m * a.lda + k, g);
+    Vec8<float>::load(A + (size_t)m * a.lda + a.K + k, u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = round_to<T>(glu_clamp_in(g[j], u[j], a.p0, a.p1));
+    return;
+  }
+  if (IN == IN_BIAS_XIELU) {
+    float bv[8];
+    Vec8<float>::load(A + (size_t)m * a.lda + k, x);
+    if (a.in_bias) Vec8<float>::load(a.in_bias + k, bv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) x[j] = round_to<T>(xielu_in(x[j] + (a.in_bias ? bv[j] : 0.f), a.p0, a.p1));
+    return;
+  }
   const int r = a.src_row[m];
-  const float w = a.src_scale[r];
+  const float w = a.src_scale ? a.src_scale[r] : 1.0f;
   Vec8<float>::load(A + (size_t)(r / a.src_div) * a.lda + k, x);
 #pragma unroll
   for (int j = 0; j < 8; ++j) x[j] = round_to<T>(w * x[j]);
@@ -403,26 +431,36 @@ extern "C" int mrs_hyb_gemm(const void *A, const void *W, float *C, int M, int N
   return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemm: launch failed");
 }
 
-/* in_mode: 0 plain (A in dtype), 1 GLU (A = f32 [M, 2 K] gate | up), 2 scaled rows (A = f32 source rows; row m = src_scale[r] * A[r / src_div], r = src_row[m]) */
-extern "C" int mrs_hyb_gemv(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
-                            const int *row_group, long long wstride, int in_mode, const int *src_row, const float *src_scale, int src_div, void *stream) {
+/* in_mode: 0 plain (A in dtype), 1 GLU (A = f32 [M, 2 K] gate | up), 2 scaled rows (A = f32 source rows; row m = src_scale[r] * A[r / src_div], r = src_row[m]; no
+ * src_scale: the rows are gathered as they are), 3 clamped GLU (A = f32 [M, 2 K]; p0 = limit, p1 = the sigmoid's factor), 4 xIELU(A + in_bias) (p0, p1 = its coefficients) */
+extern "C" int mrs_hyb_gemv_act(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate, const int *row_group,
+                                long long wstride, int in_mode, const int *src_row, const float *src_scale, int src_div, const float *in_bias, float p0, float p1, void *stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2) || in_mode < 0 || in_mode > 2) return fail("mrs_hyb_gemv: bad shape / dtype / input mode");
-  if (in_mode == 1 && lda < 2 * K) return fail("mrs_hyb_gemv: the gate | up operand needs rows of 2 K values");
-  if (in_mode == 2 && (!src_row || !src_scale || src_div <= 0)) return fail("mrs_hyb_gemv: scaled rows need their source table");
+  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2) || in_mode < 0 || in_mode > 4) return fail("mrs_hyb_gemv: bad shape / dtype / input mode");
+  if ((in_mode == 1 || in_mode == 3) && lda < 2 * K) return fail("mrs_hyb_gemv: the gate | up operand needs rows of 2 K values");
+  if (in_mode == 2 && (!src_row || src_div <= 0)) return fail("mrs_hyb_gemv: gathered rows need their source table");
   if (!row_group && M > 8) return fail("mrs_hyb_gemv: at most 8 rows share a weight");
   if (row_group && M > 65535) return fail("mrs_hyb_gemv: too many rows");
   const int esz = dtype == 1 ? 2 : 4;
   GemvArgs a{A, W, C, M, N, K, lda, ldw, ldc, accumulate, row_group, wstride,
-             (K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0) ? 1 : 0, src_row, src_scale, src_div};
+             (K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0 &&
+              (!in_bias || ((uintptr_t)in_bias % 16) == 0)) ? 1 : 0, src_row, src_scale, src_div, in_bias, p0, p1};
   dim3 grid((N + 3) / 4, row_group ? M : 1);
   hipStream_t s = (hipStream_t)stream;
 #define MRS_GEMV_(T, MR, IN) hipLaunchKernelGGL((gemv_rows_kernel<T, MR, IN>), grid, dim3(256), 0, s, a)
-#define MRS_GEMV(T, MR) do { if (in_mode == 0) MRS_GEMV_(T, MR, IN_PLAIN); else if (in_mode == 1) MRS_GEMV_(T, MR, IN_GLU); else MRS_GEMV_(T, MR, IN_SCALED); } while (0)
+#define MRS_GEMV(T, MR) do { if (in_mode == 0) MRS_GEMV_(T, MR, IN_PLAIN); else if (in_mode == 1) MRS_GEMV_(T, MR, IN_GLU); else if (in_mode == 2) MRS_GEMV_(T, MR, IN_SCALED); \
+                             else if (in_mode == 3) MRS_GEMV_(T, MR, IN_GLU_CLAMP); else MRS_GEMV_(T, MR, IN_BIAS_XIELU); } while (0)
   const int mr = row_group ? 1 : M;
   if (dtype == 1) { if (mr <= 1) MRS_GEMV(mrs::bf16_t, 1); else if (mr <= 2) MRS_GEMV(mrs::bf16_t, 2); else if (mr <= 4) MRS_GEMV(mrs::bf16_t, 4); else MRS_GEMV(mrs::bf16_t, 8); }
   else { if (mr <= 1) MRS_GEMV(float, 1); else if (mr <= 2) MRS_GEMV(float, 2); else if (mr <= 4) MRS_GEMV(float, 4); else MRS_GEMV(float, 8); }
 #undef MRS_GEMV
 #undef MRS_GEMV_
   return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemv: launch failed");
+}
+
+extern "C" int mrs_hyb_gemv(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
+                            const int *row_group, long long wstride, int in_mode, const int *src_row, const float *src_scale, int src_div, void *stream) {
+  if (in_mode < 0 || in_mode > 2) return fail("mrs_hyb_gemv: bad shape / dtype / input mode");
+  if (in_mode == 2 && !src_scale) return fail("mrs_hyb_gemv: scaled rows need their source table");
+  return mrs_hyb_gemv_act(A, W, C, M, N, K, lda, ldw, ldc, dtype, accumulate, row_group, wstride, in_mode, src_row, src_scale, src_div, nullptr, 0.f, 0.f, stream);
 }

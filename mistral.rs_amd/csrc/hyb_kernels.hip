@@ -673,10 +673,11 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
 }
 
 // ---------------------------------------------------------------------------------- mixture of experts: routing, dispatch, gather, GLU, combine
-// Router: one workgroup per row.  logits z_e = w_e . h in f32 (a wave per expert, lanes over the width, butterfly sum), score = sigmoid(z); the `top` largest (ties: the
-// lower index), weights = the scores, un-renormalised; row E of the weight (when has_gate) is the shared expert's gate: gate[t] = sigmoid(w_E . h).
-__global__ void __launch_bounds__(1024) route_sigmoid_topk_kernel(const float *__restrict__ h, const float *__restrict__ wr, int W, int E, int top, int has_gate, int *__restrict__ ids,
-                                                                  float *__restrict__ wts, float *__restrict__ gate) {
+// Router: one workgroup per row.  logits z_e = w_e . h in f32 (a wave per expert, lanes over the width, butterfly sum); the `top` largest (ties: the lower index).
+// SOFTMAX false: score = sigmoid(z), weights = the scores, un-renormalised; row E of the weight (when has_gate) is the shared expert's gate: gate[t] = sigmoid(w_E . h).
+// SOFTMAX true: score = softmax(z) over ALL experts, weights = out_scale * the chosen scores, un-renormalised.
+template <bool SOFTMAX> __global__ void __launch_bounds__(1024) route_topk_kernel(const float *__restrict__ h, const float *__restrict__ wr, int W, int E, int top, int has_gate,
+                                                                                  int *__restrict__ ids, float *__restrict__ wts, float *__restrict__ gate, float out_scale) {
   extern __shared__ float z[];  // [E + 1]
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float *hr = h + (size_t)t * W;
@@ -699,6 +700,15 @@ __global__ void __launch_bounds__(1024) route_sigmoid_topk_kernel(const float *_
   __syncthreads();
   if (wave != 0) return;
   if (has_gate && lane == 0) gate[t] = sigmoid_f(z[E]);
+  float zmax = 0.f, zden = 1.f;
+  if (SOFTMAX) {
+    float mx = -FLT_MAX;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    zmax = wave_max(mx);
+    float den = 0.f;
+    for (int e = lane; e < E; e += 64) den += expf(z[e] - zmax);
+    zden = wave_sum(den);
+  }
   for (int k = 0; k < top; ++k) {
     float bv = -FLT_MAX;
     int be = 0x7fffffff;
@@ -712,7 +722,7 @@ __global__ void __launch_bounds__(1024) route_sigmoid_topk_kernel(const float *_
     }
     if (lane == 0) {
       ids[(size_t)t * top + k] = be;
-      wts[(size_t)t * top + k] = sigmoid_f(bv);
+      wts[(size_t)t * top + k] = SOFTMAX ? out_scale * (expf(bv - zmax) / zden) : sigmoid_f(bv);
     }
     if ((be & 63) == lane) z[be] = -FLT_MAX;  // taken: written by the lane that reads this entry in the next round (every lane holds the same `be` after the butterfly)
   }
@@ -763,7 +773,7 @@ __global__ void __launch_bounds__(256) moe_dispatch_kernel(const int *__restrict
 template <class T> __global__ void __launch_bounds__(256) moe_gather_kernel(const float *__restrict__ h32, const int *__restrict__ sorted_route, const float *__restrict__ wts, int top,
                                                                             T *__restrict__ out, int W) {
   const int i = blockIdx.x, r = sorted_route[i], t = r / top;
-  const float w = wts[r];
+  const float w = wts ? wts[r] : 1.0f;  // no weights: the rows are gathered as they are (the route's weight multiplies the expert's output instead)
   for (int c = threadIdx.x; c < W; c += 256) out[(size_t)i * W + c] = from_f<T>(w * h32[(size_t)t * W + c]);
 }
 // silu(gate) * up; gu [rows, 2 ff] = gate | up
@@ -774,15 +784,104 @@ template <class T> __global__ void __launch_bounds__(256) glu_silu_kernel(const 
   const float gv = gu[r * 2 * ff + c], uv = gu[r * 2 * ff + ff + c];
   out[i] = from_f<T>(silu_f(gv) * uv);
 }
-// x[t] += sum_k d[route_pos[t top + k]] + gate[t] * shared[t]
+// g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1); gu [rows, 2 ff] = gate | up
+__device__ __forceinline__ float glu_clamped_f(float gv, float uv, float limit, float alpha) {
+  const float g = fminf(gv, limit), u = fminf(fmaxf(uv, -limit), limit);
+  return g * sigmoid_f(alpha * g) * (u + 1.0f);
+}
+template <class T> __global__ void __launch_bounds__(256) glu_clamped_kernel(const float *__restrict__ gu, T *__restrict__ out, int rows, int ff, float limit, float alpha) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)rows * ff) return;
+  const size_t r = i / ff, c = i % ff;
+  out[i] = from_f<T>(glu_clamped_f(gu[r * 2 * ff + c], gu[r * 2 * ff + ff + c], limit, alpha));
+}
+// xIELU of (u + bias): z > 0: ap z^2 + z / 2;  z <= 0: an (e^z - 1 - z) + z / 2      (ap = softplus(p), an = 1 / 2 + softplus(q), both evaluated by the caller)
+__device__ __forceinline__ float xielu_f(float z, float ap, float an) { return z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(an, expm1f(z) - z, 0.5f * z); }
+template <class T> __global__ void __launch_bounds__(256) bias_xielu_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ bias, T *__restrict__ out, int rows, int ff,
+                                                                            float ap, float an) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)rows * ff) return;
+  const size_t r = i / ff, c = i % ff;
+  out[i] = from_f<T>(xielu_f(u[r * ldu + c] + (bias ? bias[c] : 0.f), ap, an));
+}
+// out[t] (+)= sum_k w_k d[route_pos[t top + k]] + gate[t] * shared[t]        (w_k = wts[t top + k], or 1 without weights: the experts' inputs were scaled instead)
 __global__ void __launch_bounds__(256) moe_combine_kernel(float *__restrict__ x, const float *__restrict__ d, const int *__restrict__ route_pos, int top, const float *__restrict__ shared,
-                                                          const float *__restrict__ gate, int W) {
+                                                          const float *__restrict__ gate, int W, const float *__restrict__ wts, int accumulate) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += 256) {
     float acc = 0.f;
-    for (int k = 0; k < top; ++k) acc += d[(size_t)route_pos[(size_t)t * top + k] * W + c];
+    for (int k = 0; k < top; ++k) {
+      const float v = d[(size_t)route_pos[(size_t)t * top + k] * W + c];
+      acc = wts ? fmaf(wts[(size_t)t * top + k], v, acc) : acc + v;
+    }
     if (shared) acc += (gate ? gate[t] : 1.0f) * shared[(size_t)t * W + c];
-    x[(size_t)t * W + c] += acc;
+    x[(size_t)t * W + c] = accumulate ? x[(size_t)t * W + c] + acc : acc;
+  }
+}
+
+// ---------------------------------------------------------------------------------- layer norm with weight and bias: (v - mean) / sqrt(mean((v - mean)^2) + eps) * w + b
+// v = x (+ in_bias): the bias of the product that made x.  The result goes to out (T) and / or out32, and / or is ADDED to resid (the f32 residual stream: norms after a sublayer).
+template <class T> __global__ void __launch_bounds__(256) layernorm_kernel(const float *__restrict__ x, int ldx, const float *__restrict__ in_bias, const float *__restrict__ w,
+                                                                           const float *__restrict__ b, T *__restrict__ out, float *__restrict__ out32, float *__restrict__ resid, int ldr,
+                                                                           int width, float eps) {
+  __shared__ float red[4];
+  extern __shared__ float row[];
+  const int t = blockIdx.x;
+  const float *xr = x + (size_t)t * ldx;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = xr[c] + (in_bias ? in_bias[c] : 0.f);
+    row[c] = v;
+    s += v;
+  }
+  const float mean = block_sum_256(s, red) / (float)width;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float dv = row[c] - mean;
+    q = fmaf(dv, dv, q);
+  }
+  const float inv = 1.0f / sqrtf(block_sum_256(q, red) / (float)width + eps);
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float y = (row[c] - mean) * inv * w[c] + (b ? b[c] : 0.f);
+    if (out) out[(size_t)t * width + c] = from_f<T>(y);
+    if (out32) out32[(size_t)t * width + c] = y;
+    if (resid) resid[(size_t)t * ldr + c] += y;
+  }
+}
+
+// ---------------------------------------------------------------------------------- projection biases, query temperature, K / V page write (no norm, no rotation)
+// q <- (q + qb) * (1 + coef ln(floor((pos + 1) / every) + 1)) in f32, rounded once to T; k + kb and v + vb go to the page slot of the row (no k_cache: the layer reads another
+// layer's pages and has no key / value columns)
+struct QkvBiasArgs {
+  const float *qkv;   // [rows, ld]: q [H * D] | k [G * D] | v [G * Dv] | ...
+  const float *qb, *kb, *vb;  // nullable
+  const int *tok_pos;
+  const long long *slot_mapping;
+  void *q_out, *k_cache, *v_cache;
+  int ld, H, G, D, Dv, block_size, temp_every;
+  float temp_coef;
+};
+template <class T> __global__ void __launch_bounds__(256) qkv_bias_temp_cache_kernel(QkvBiasArgs a) {
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int nq = a.H * a.D, nk = a.G * a.D, nv = a.G * a.Dv;
+  const float *q = a.qkv + (size_t)t * a.ld;
+  float f = 1.0f;
+  if (a.temp_every > 0) f = 1.0f + a.temp_coef * logf((float)((a.tok_pos[t] + 1) / a.temp_every + 1));
+  T *qo = (T *)a.q_out + (size_t)t * nq;
+  for (int c = tid; c < nq; c += 256) qo[c] = from_f<T>((q[c] + (a.qb ? a.qb[c] : 0.f)) * f);
+  if (!a.k_cache) return;
+  const long long slot = a.slot_mapping[t];
+  if (slot < 0) return;
+  const long long blk = slot / a.block_size;
+  const int off = (int)(slot % a.block_size);
+  const float *k = q + nq, *v = k + nk;
+  for (int e = tid; e < nk; e += 256) {
+    const int g = e / a.D, d = e % a.D;
+    ((T *)a.k_cache)[(((size_t)blk * a.G + g) * a.block_size + off) * a.D + d] = from_f<T>(k[e] + (a.kb ? a.kb[e] : 0.f));
+  }
+  for (int e = tid; e < nv; e += 256) {
+    const int g = e / a.Dv, d = e % a.Dv;
+    ((T *)a.v_cache)[(((size_t)blk * a.G + g) * a.block_size + off) * a.Dv + d] = from_f<T>(v[e] + (a.vb ? a.vb[e] : 0.f));
   }
 }
 __global__ void __launch_bounds__(256) gather_rows_kernel(const float *__restrict__ x, const int *__restrict__ idx, float *__restrict__ out, int W) {
@@ -929,8 +1028,16 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
 extern "C" int mrs_hyb_route_sigmoid_topk(const float *h, const float *wr, int rows, int W, int E, int top, int has_gate, int *ids, float *wts, float *gate, void *stream) {
   if (rows <= 0) return 0;
   if (top < 1 || top > E || E > 8192) return fail("mrs_hyb_route_sigmoid_topk: 1 <= top <= experts <= 8192");
-  hipLaunchKernelGGL(route_sigmoid_topk_kernel, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, has_gate, ids, wts, gate);
+  hipLaunchKernelGGL(route_topk_kernel<false>, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, has_gate, ids, wts, gate, 1.0f);
   return ok_or("mrs_hyb_route_sigmoid_topk");
+}
+
+/* softmax over all experts, the `top` largest, weights = scale * score (not renormalised over the chosen) */
+extern "C" int mrs_hyb_route_softmax_topk(const float *h, const float *wr, int rows, int W, int E, int top, float scale, int *ids, float *wts, void *stream) {
+  if (rows <= 0) return 0;
+  if (top < 1 || top > E || E > 8192) return fail("mrs_hyb_route_softmax_topk: 1 <= top <= experts <= 8192");
+  hipLaunchKernelGGL(route_topk_kernel<true>, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, 0, ids, wts, (float *)nullptr, scale);
+  return ok_or("mrs_hyb_route_softmax_topk");
 }
 
 extern "C" int mrs_hyb_moe_dispatch(const int *ids, int R, int E, int *bounds, int *sorted_route, int *route_pos, int *sorted_expert, void *stream) {
@@ -959,8 +1066,61 @@ extern "C" int mrs_hyb_glu_silu(const float *gu, void *out, int rows, int ff, in
 
 extern "C" int mrs_hyb_moe_combine(float *x, const float *d, const int *route_pos, int top, const float *shared, const float *gate, int rows, int W, void *stream) {
   if (rows <= 0) return 0;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(rows), dim3(256), 0, S_(stream), x, d, route_pos, top, shared, gate, W);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(rows), dim3(256), 0, S_(stream), x, d, route_pos, top, shared, gate, W, (const float *)nullptr, 1);
   return ok_or("mrs_hyb_moe_combine");
+}
+
+/* out[t] (+)= sum_k wts[t top + k] * d[route_pos[t top + k]] + shared[t] (shared nullable) */
+extern "C" int mrs_hyb_moe_combine_weighted(float *out, const float *d, const int *route_pos, const float *wts, int top, const float *shared, int rows, int W, int accumulate,
+                                            void *stream) {
+  if (rows <= 0) return 0;
+  if (!wts) return fail("mrs_hyb_moe_combine_weighted: the route weights are missing");
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(rows), dim3(256), 0, S_(stream), out, d, route_pos, top, shared, (const float *)nullptr, W, wts, accumulate);
+  return ok_or("mrs_hyb_moe_combine_weighted");
+}
+
+extern "C" int mrs_hyb_glu_clamped(const float *gu, void *out, int rows, int ff, float limit, float alpha, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  const unsigned blocks = (unsigned)(((size_t)rows * ff + 255) / 256);
+  if (dtype == 1) hipLaunchKernelGGL(glu_clamped_kernel<mrs::bf16_t>, dim3(blocks), dim3(256), 0, S_(stream), gu, (mrs::bf16_t *)out, rows, ff, limit, alpha);
+  else if (dtype == 2) hipLaunchKernelGGL(glu_clamped_kernel<float>, dim3(blocks), dim3(256), 0, S_(stream), gu, (float *)out, rows, ff, limit, alpha);
+  else return fail("mrs_hyb_glu_clamped: dtype");
+  return ok_or("mrs_hyb_glu_clamped");
+}
+
+/* out (dtype) = xIELU(u + bias); ap = softplus(p), an = 1 / 2 + softplus(q) of the layer's two activation numbers */
+extern "C" int mrs_hyb_bias_xielu(const float *u, int ldu, const float *bias, void *out, int rows, int ff, float ap, float an, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  const unsigned blocks = (unsigned)(((size_t)rows * ff + 255) / 256);
+  if (dtype == 1) hipLaunchKernelGGL(bias_xielu_kernel<mrs::bf16_t>, dim3(blocks), dim3(256), 0, S_(stream), u, ldu, bias, (mrs::bf16_t *)out, rows, ff, ap, an);
+  else if (dtype == 2) hipLaunchKernelGGL(bias_xielu_kernel<float>, dim3(blocks), dim3(256), 0, S_(stream), u, ldu, bias, (float *)out, rows, ff, ap, an);
+  else return fail("mrs_hyb_bias_xielu: dtype");
+  return ok_or("mrs_hyb_bias_xielu");
+}
+
+/* Layer norm of every row of x (+ in_bias): out (dtype, nullable), out32 (nullable), resid (nullable, f32 [rows, ldr]): resid += the normed row */
+extern "C" int mrs_hyb_layernorm(const float *x, int ldx, const float *in_bias, const float *w, const float *b, void *out, float *out32, float *resid, int ldr, int rows, int width,
+                                 float eps, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  if (width <= 0 || width > 15000) return fail("mrs_hyb_layernorm: 1 .. 15000 values per row");
+  const size_t lds = (size_t)width * 4;
+  if (dtype == 1) hipLaunchKernelGGL(layernorm_kernel<mrs::bf16_t>, dim3(rows), dim3(256), lds, S_(stream), x, ldx, in_bias, w, b, (mrs::bf16_t *)out, out32, resid, ldr, width, eps);
+  else if (dtype == 2) hipLaunchKernelGGL(layernorm_kernel<float>, dim3(rows), dim3(256), lds, S_(stream), x, ldx, in_bias, w, b, (float *)out, out32, resid, ldr, width, eps);
+  else return fail("mrs_hyb_layernorm: dtype");
+  return ok_or("mrs_hyb_layernorm");
+}
+
+/* temp_every <= 0: no query temperature.  k_cache null: the rows carry no key / value columns (a layer that reads another layer's pages) */
+extern "C" int mrs_hyb_qkv_bias_temp_cache(const float *qkv, int ld, const float *qb, const float *kb, const float *vb, const int *tok_pos, const long long *slot_mapping, void *q_out,
+                                           void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int block_size, float temp_coef, int temp_every, int dtype,
+                                           void *stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || (k_cache && !v_cache)) return fail("mrs_hyb_qkv_bias_temp_cache: head sizes (heads % kv_heads == 0)");
+  QkvBiasArgs a{qkv, qb, kb, vb, tok_pos, slot_mapping, q_out, k_cache, v_cache, ld, H, G, D, Dv, block_size, temp_every, temp_coef};
+  if (dtype == 1) hipLaunchKernelGGL(qkv_bias_temp_cache_kernel<mrs::bf16_t>, dim3(rows), dim3(256), 0, S_(stream), a);
+  else if (dtype == 2) hipLaunchKernelGGL(qkv_bias_temp_cache_kernel<float>, dim3(rows), dim3(256), 0, S_(stream), a);
+  else return fail("mrs_hyb_qkv_bias_temp_cache: dtype");
+  return ok_or("mrs_hyb_qkv_bias_temp_cache");
 }
 
 extern "C" int mrs_hyb_gather_rows(const float *x, const int *idx, float *out, int n, int W, void *stream) {

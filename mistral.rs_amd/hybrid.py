@@ -1,6 +1,8 @@
 """Layer-list ("hybrid") decoders served in their checkpoint dtype: every layer is `x += mixer(norm(x))` then optionally `x += feed_forward(norm(x))`, the mixer being
-one of the registered kinds (`MIXERS`: state-space-duality recurrence, paged attention with a sliding window and kept first tokens), the feed-forward one of
-`FEED_FORWARDS` (sigmoid-routed experts with a gated shared expert).  The Gekilix architecture (config.json `"architecture": "Gekilix"`) is one such list.
+one of the registered kinds (`MIXERS`: state-space-duality recurrence, paged softmax attention with a sliding window and kept first tokens, paged sigmoid attention with a
+distance bias and mixed head scores), the feed-forward one of `FEED_FORWARDS` (sigmoid-routed experts with a gated shared expert, softmax-routed clamped-GLU experts, a
+dense xIELU layer).  The norms are one-plus RMS norms before every sublayer, or layer norms with bias before AND after every sublayer (`HybridSpec.norm`, `post_norms`).
+The Gekilix and Sobunex architectures (config.json `"architecture"`) are two such lists.
 
 The step function is `HybridDecoder.forward_batch(batch)`: ONE ragged batch -- prompt portions of any length next to single decoded tokens -- through the HIP kernels of
 csrc/hyb_kernels.hip and csrc/hyb_gemm.hip (C ABI, this process's current stream; PyTorch owns buffers and the stream, nothing else).  What the sequences carry between
@@ -41,8 +43,16 @@ _SIGS = {
     "mrs_hyb_glu_silu": [_vp, _vp, _i, _i, _i, _vp],
     "mrs_hyb_moe_combine": [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp],
     "mrs_hyb_gather_rows": [_vp, _vp, _vp, _i, _i, _vp],
+    "mrs_hyb_route_softmax_topk": [_vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _vp],
+    "mrs_hyb_moe_combine_weighted": [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp],
+    "mrs_hyb_glu_clamped": [_vp, _vp, _i, _i, _f, _f, _i, _vp],
+    "mrs_hyb_bias_xielu": [_vp, _i, _vp, _vp, _i, _i, _f, _f, _i, _vp],
+    "mrs_hyb_layernorm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp],
+    "mrs_hyb_qkv_bias_temp_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp],
+    "mrs_hyb_paged_talk_sigmoid_attn": [_vp] * 9 + [_i, _vp] + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _vp],
     "mrs_hyb_gemm": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _l, _i, _vp],
     "mrs_hyb_gemv": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp],
+    "mrs_hyb_gemv_act": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp, _f, _f, _vp],
 }
 _fns: dict = {}
 _step_stream: Optional[int] = None   # the stream handle of the step in progress (looked up once per forward_batch, not once per launch)
@@ -55,7 +65,7 @@ def _call(name: str, *args) -> None:
         fn = _fns[name] = _lib.sym("hybrid", name, _SIGS[name], C.c_int)
     conv = [a.data_ptr() if isinstance(a, torch.Tensor) else a for a in args]
     if fn(*conv, _step_stream if _step_stream is not None else torch.cuda.current_stream().cuda_stream) != 0:
-        err = _lib.sym("hybrid", "mrs_hyb_gemm_last_error" if "gem" in name else "mrs_hyb_last_error", [], C.c_char_p)()
+        err = _lib.sym("hybrid", "mrs_hyb_gemm_last_error" if "gem" in name else ("mrs_hyb_talk_last_error" if "talk" in name else "mrs_hyb_last_error"), [], C.c_char_p)()
         raise ValueError((err or b"").decode() or name)
 
 
@@ -81,6 +91,7 @@ class RaggedBatch:
     seg_row0: Optional[torch.Tensor] = None    # i32 [segments]  first row
     seg_len: Optional[torch.Tensor] = None     # i32 [segments]
     ent_seg0: Optional[torch.Tensor] = None    # i32 [entries + 1]  first segment of every entry, then the total
+    seg_rows: int = 0                          # rows of the longest segment (1: every entry brings one decoded token)
 
     SEGMENT = int(os.environ.get("MRS_HYB_SEGMENT", "64"))   # rows per segment
 
@@ -136,7 +147,7 @@ class RaggedBatch:
             dv.append(dev_ints[o:o + n])
             o += n
         return RaggedBatch(T, S, mb, dv[0], dv[1], dv[2], dv[3], dv[4], dv[5], dv[6].view(S, mb), torch.from_numpy(slots).to(device),
-                           torch.tensor(want, dtype=torch.int32, device=device), nseg, dv[7], dv[8], dv[9], dv[10])
+                           torch.tensor(want, dtype=torch.int32, device=device), nseg, dv[7], dv[8], dv[9], dv[10], max(1, min(L, max(lens, default=1))))
 
 
 # ------------------------------------------------------------------------------------------------------------------ layer descriptions
@@ -174,6 +185,20 @@ class AttentionSpec:
 
 
 @dataclass
+class TalkAttentionSpec:
+    """Sigmoid attention with a distance bias, mixed head scores, a query temperature and a per-head output gate (TalkSigmoidAttention)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0            # 0: every earlier token
+    temp_coef: float = 0.0     # query factor 1 + temp_coef ln(floor((pos + 1) / temp_every) + 1); temp_every 0: none
+    temp_every: int = 0
+    kv_from: Optional[int] = None   # index of the layer whose K / V pages this layer reads (it has no key / value projections then)
+
+
+@dataclass
 class Mamba2Spec:
     heads: int
     vdim: int
@@ -197,13 +222,34 @@ class MoeSpec:
     top: int
     ff: int
     shared_ff: int = 0         # 0: no shared expert
+    kind = "moe"               # key into FEED_FORWARDS
+
+
+@dataclass
+class ClampedMoeSpec:
+    """Softmax-routed experts with a clamped GLU (ClampedSoftmaxMoe)."""
+    experts: int
+    top: int
+    ff: int
+    limit: float
+    route_scale: float = 1.0
+    shared_ff: int = 0         # 0: no shared expert
+    shared_limit: float = 0.0
+    kind = "moe_softmax_clamped"
+
+
+@dataclass
+class DenseSpec:
+    """down(xIELU(up h + b) ) + b (XieluFeedForward)."""
+    ff: int
+    kind = "dense_xielu"
 
 
 @dataclass
 class LayerSpec:
     kind: str
     mixer: object
-    ff: Optional[MoeSpec]
+    ff: Optional[object]       # MoeSpec | ClampedMoeSpec | DenseSpec | None
     prefix: str                # tensor-name prefix of the layer
 
 
@@ -216,6 +262,8 @@ class HybridSpec:
     embed: str = "embed"
     final_norm: str = "final.norm"
     head: str = "head"
+    norm: str = "rms_one_plus"   # "rms_one_plus": x / rms * (1 + w);  "layer": (x - mean) / sqrt(var + eps) * w + b, the bias being the tensor `<name>.b`
+    post_norms: bool = False     # every sublayer's output is normed (`norm1b` / `norm2b`) before it joins the residual stream
 
 
 def gekilix_spec(cfg: dict) -> HybridSpec:
@@ -244,8 +292,45 @@ def gekilix_spec(cfg: dict) -> HybridSpec:
     return HybridSpec(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers)
 
 
+def sobunex_spec(cfg: dict) -> HybridSpec:
+    """config.json of a Sobunex checkpoint -> the layer list: layer norms (weight and bias) before and after every sublayer, sigmoid attention mixers (some reading an
+    earlier layer's K / V pages), dense xIELU or softmax-routed clamped-GLU feed-forwards.  Every size and every model-dependent constant comes from the file."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        m = L["mixer"]
+        if L["type"] != "attention":
+            raise ValueError(f"Sobunex: unknown layer type {L['type']!r}")
+        mask, qt = m.get("mask") or {}, m.get("q_temp") or {}
+        src = m.get("kv_from")
+        if src is not None and not 0 <= int(src) < i:
+            raise ValueError(f"Sobunex: layer {i} reads the keys of layer {src}, which does not run before it")
+        mixer = TalkAttentionSpec(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), float(m["scale"]), int(mask.get("size", 0) or 0),
+                                  float(qt.get("coef", 0.0) or 0.0), int(qt.get("every", 0) or 0) if qt.get("coef") else 0, None if src is None else int(src))
+        f = L.get("mlp")
+        ff = None
+        if f:
+            if f.get("kind") == "dense":
+                ff = DenseSpec(int(f["ff"]))
+            elif f.get("kind") == "moe":
+                r, sh = f["router"], f.get("shared")
+                ff = ClampedMoeSpec(int(r["experts"]), int(r["top"]), int(f["expert"]["ff"]), float(f["expert"]["limit"]), float(r.get("scale", 1.0)),
+                                    int(sh["ff"]) if sh else 0, float(sh["limit"]) if sh else 0.0)
+            else:
+                raise ValueError(f"Sobunex: unknown feed-forward kind {f.get('kind')!r}")
+        layers.append(LayerSpec("talk_attention", mixer, ff, f"l{i}."))
+    for i, ls in enumerate(layers):
+        j = ls.mixer.kv_from
+        if j is not None:
+            o = layers[j].mixer
+            if o.kv_from is not None or (o.kv_heads, o.dim, o.vdim) != (ls.mixer.kv_heads, ls.mixer.dim, ls.mixer.vdim):
+                raise ValueError(f"Sobunex: layer {i} cannot read the keys and values of layer {j} (no projections of its own there, or other head sizes)")
+    return HybridSpec(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, norm="layer", post_norms=True)
+
+
 # ------------------------------------------------------------------------------------------------------------------ mixers and feed-forwards
 class _Module:
+    out_bias = None            # f32 bias of the module's last product, left to the caller (a norm that follows adds it while it reads the product)
+
     def __init__(self, model: "HybridDecoder"):
         self.m = model
 
@@ -277,7 +362,10 @@ class Mamba2Mixer(_Module):
         if tuple(self.w_in.shape) != (n_in, self.m.spec.width) or tuple(self.conv_w.shape) != (s.conv_channels, s.conv):
             raise ValueError(f"{p}: tensor shapes do not match the mixer's sizes")
 
-    def forward(self, h, x, b: RaggedBatch):
+    def carried(self):
+        return (self.conv_state, self.ssm_state)
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
         s, m = self.s, self.m
         T = b.rows
         u = m.linear(h, self.w_in)                                         # f32 [T, z | x B C | dt]
@@ -293,7 +381,7 @@ class Mamba2Mixer(_Module):
         _call("mrs_hyb_ssd_scan", xbc, u, self.dt_bias, self.A_log, self.D, self.ssm_state, y, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0,
               steps, carry, decay, T, b.entries, b.segments, s.conv_channels, u.stride(0), s.inner + s.conv_channels, s.heads, s.vdim, s.state, s.groups)
         yn = m.norm(y, self.norm, one_plus=False, parts=s.norm_groups, gate=u)   # y * silu(z) (z = the first `inner` columns of u), then the grouped norm
-        m.linear(yn, self.w_o, out=x, accumulate=True)
+        m.linear(yn, self.w_o, out=x, accumulate=accumulate)
 
     def state_bytes_per_slot(self) -> int:
         return 4 * (self.conv_state[0].numel() + self.ssm_state[0].numel())
@@ -322,7 +410,13 @@ class WindowAttention(_Module):
         self.q_norm = self.w(get, p + "q.norm", False) if s.qk_norm else None
         self.k_norm = self.w(get, p + "k.norm", False) if s.qk_norm else None
 
-    def forward(self, h, x, b: RaggedBatch):
+    def carried(self):
+        return (self.k_cache, self.v_cache)
+
+    def kv_bytes_per_token(self) -> int:
+        return self.k_cache.element_size() * self.s.kv_heads * (self.s.dim + self.s.vdim)
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
         s, m = self.s, self.m
         T = b.rows
         qkv = m.linear(h, self.w_qkv)
@@ -332,7 +426,62 @@ class WindowAttention(_Module):
         o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
         _call("mrs_hyb_paged_window_attn", q, self.k_cache, self.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size,
               b.max_blocks, s.window, s.keep_first, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
-        m.linear(o, self.w_o, out=x, accumulate=True)
+        m.linear(o, self.w_o, out=x, accumulate=accumulate)
+
+
+class TalkSigmoidAttention(_Module):
+    """q, k, v and the output projection with biases, the per-head gate logits in the same product.  No rotation: positions enter through a query temperature
+    (q *= 1 + coef ln(floor((pos + 1) / every) + 1)) and a per-head distance bias.  Head g scores key j as scale (q_g . k_j) - 2^(-8 (g + 1) / heads) (i - j); the heads'
+    scores are mixed by the [heads, heads] matrix `talk`; a key with 0 <= i - j < window weighs sigmoid(mixed + pb_h), un-normalised; head outputs are multiplied by
+    sigmoid(gate logit), then projected.  With `kv_from` the layer has no key / value projections: it reads the K / V pages of that earlier layer (same block tables)."""
+
+    def __init__(self, model, spec: TalkAttentionSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+        if spec.heads % spec.kv_heads:
+            raise ValueError(f"{prefix}: heads % kv_heads must be 0")
+        dev, bs, nb = model.device, model.block_size, model.num_blocks
+        self.k_cache = self.v_cache = None
+        if spec.kv_from is None:
+            self.k_cache = torch.zeros(nb, spec.kv_heads, bs, spec.dim, dtype=model.torch_dtype, device=dev)
+            self.v_cache = torch.zeros(nb, spec.kv_heads, bs, spec.vdim, dtype=model.torch_dtype, device=dev)
+        self.slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / spec.heads) for h in range(spec.heads)], dtype=torch.float64).to(dev, torch.float32)
+
+    def carried(self):
+        return (self.k_cache, self.v_cache) if self.k_cache is not None else ()
+
+    def kv_bytes_per_token(self) -> int:
+        return self.k_cache.element_size() * self.s.kv_heads * (self.s.dim + self.s.vdim) if self.k_cache is not None else 0
+
+    def load(self, get):
+        s, p, own = self.s, self.p, self.s.kv_from is None
+        names = ["q", "k", "v"] if own else ["q"]
+        parts = [get(p + n) for n in names] + [get(p + "g")]
+        want = [s.heads * s.dim, s.kv_heads * s.dim, s.kv_heads * s.vdim][:len(names)] + [s.heads]
+        if [t.shape[0] for t in parts] != want or any(t.shape[1] != self.m.spec.width for t in parts):
+            raise ValueError(f"{p}: projection shapes do not match the mixer's sizes")
+        self.w_in = torch.cat(parts, 0).to(self.m.device, self.m.torch_dtype).contiguous()     # [q | k | v | gate, W]
+        self.gate_col = sum(want[:-1])
+        self.qb = self.w(get, p + "q.b", False)
+        self.kb = self.w(get, p + "k.b", False) if own else None
+        self.vb = self.w(get, p + "v.b", False) if own else None
+        self.w_o, self.out_bias = self.w(get, p + "o", True), self.w(get, p + "o.b", False)
+        self.talk, self.pb = self.w(get, p + "talk", False), self.w(get, p + "pb", False)
+        if tuple(self.talk.shape) != (s.heads, s.heads) or self.pb.numel() != s.heads or tuple(self.w_o.shape) != (self.m.spec.width, s.heads * s.vdim):
+            raise ValueError(f"{p}: head-mixing / output shapes do not match the mixer's sizes")
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T = b.rows
+        u = m.linear(h, self.w_in)                                         # f32 [T, q | k | v | gate logits]
+        q = torch.empty(T, s.heads * s.dim, dtype=m.torch_dtype, device=m.device)
+        _call("mrs_hyb_qkv_bias_temp_cache", u, u.stride(0), self.qb, self.kb, self.vb, b.tok_pos, b.slot_mapping, q, self.k_cache, self.v_cache, T, s.heads, s.kv_heads,
+              s.dim, s.vdim, m.block_size, s.temp_coef, s.temp_every, m.dt)
+        src = self if s.kv_from is None else m.layers[s.kv_from].mixer      # that layer ran earlier in this step: its pages hold this step's rows already
+        o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
+        _call("mrs_hyb_paged_talk_sigmoid_attn", q, src.k_cache, src.v_cache, b.block_tables, b.tok_pos, self.talk, self.pb, self.slopes, u[:, self.gate_col:], u.stride(0), o,
+              T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, b.max_blocks, s.window, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, b.seg_rows)
+        m.linear(o, self.w_o, out=x, accumulate=accumulate)
 
 
 class SigmoidMoe(_Module):
@@ -357,9 +506,11 @@ class SigmoidMoe(_Module):
             self.ws_down = self.w(get, p + "shared.down", True)
         self.w_router = torch.cat(rows, 0).to(dev, torch.float32).contiguous()   # [E (+ 1), W] f32: router rows, then the shared expert's gate row
 
-    def forward(self, h, h32, x, b: RaggedBatch):
+    def forward(self, h, h32, x, b: RaggedBatch, accumulate: bool = True):
         s, m = self.s, self.m
         T, W, dev = b.rows, m.spec.width, m.device
+        if not accumulate:
+            x.zero_()
         R = T * s.top
         ids = torch.empty(R, dtype=torch.int32, device=dev)
         wts = torch.empty(R, dtype=torch.float32, device=dev)
@@ -395,16 +546,106 @@ class SigmoidMoe(_Module):
         _call("mrs_hyb_moe_combine", x, d, route_pos, s.top, sh, gate, T, W)
 
 
-MIXERS: Dict[str, Callable] = {"mamba2": Mamba2Mixer, "attention": WindowAttention}
-FEED_FORWARDS: Dict[str, Callable] = {"moe": SigmoidMoe}
+class ClampedSoftmaxMoe(_Module):
+    """Router logits in f32, scores = softmax over all experts, the `top` largest; weights = route_scale * score, un-renormalised, on the experts' OUTPUTS.  Expert (no
+    biases): g = min(gate h, limit), u = clamp(up h, -limit, limit), down(g sigmoid(1.702 g) (u + 1)); a shared expert of the same form (its own size and limit) runs for
+    every row with weight 1.  All experts of a step run as grouped products over expert-sorted rows."""
+    ALPHA = 1.702
+
+    def __init__(self, model, spec: ClampedMoeSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+
+    def load(self, get):
+        s, p, m = self.s, self.p, self.m
+        dev, dt = m.device, m.torch_dtype
+        self.w_gu = torch.stack([torch.cat([get(f"{p}e{e}.gate"), get(f"{p}e{e}.up")], 0) for e in range(s.experts)]).to(dev, dt).contiguous()   # [E, 2 ff, W]
+        self.w_down = torch.stack([get(f"{p}e{e}.down") for e in range(s.experts)]).to(dev, dt).contiguous()                                      # [E, W, ff]
+        self.w_router = self.w(get, p + "router", False)
+        if tuple(self.w_gu.shape[1:]) != (2 * s.ff, m.spec.width) or tuple(self.w_router.shape) != (s.experts, m.spec.width):
+            raise ValueError(f"{p}: expert / router shapes do not match the layer's sizes")
+        if s.shared_ff:
+            self.ws_gu = torch.cat([get(p + "shared.gate"), get(p + "shared.up")], 0).to(dev, dt).contiguous()
+            self.ws_down = self.w(get, p + "shared.down", True)
+            if tuple(self.ws_gu.shape) != (2 * s.shared_ff, m.spec.width):
+                raise ValueError(f"{p}: shared expert shapes do not match the layer's sizes")
+
+    def forward(self, h, h32, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T, W, dev = b.rows, m.spec.width, m.device
+        R = T * s.top
+        ids = torch.empty(R, dtype=torch.int32, device=dev)
+        wts = torch.empty(R, dtype=torch.float32, device=dev)
+        _call("mrs_hyb_route_softmax_topk", h32, self.w_router, T, W, s.experts, s.top, s.route_scale, ids, wts)
+        meta = torch.empty(s.experts + 1 + 3 * R, dtype=torch.int32, device=dev)
+        bounds, sorted_route, route_pos, sorted_expert = meta[:s.experts + 1], meta[s.experts + 1:][:R], meta[s.experts + 1 + R:][:R], meta[s.experts + 1 + 2 * R:][:R]
+        _call("mrs_hyb_moe_dispatch", ids, R, s.experts, bounds, sorted_route, route_pos, sorted_expert)
+        f32 = dict(dtype=torch.float32, device=dev)
+        if R <= m.GROUPED_GEMV_ROWS:
+            # decode-sized steps: every route streams its expert's slabs; the row gather and the clamped GLU happen in the consuming product's operand load (same roundings)
+            gu = torch.empty(R, 2 * s.ff, **f32)
+            m.gemv_act(h32, self.w_gu, gu, R, 2 * s.ff, W, h32.stride(0), W, sorted_expert, self.w_gu.stride(0), 2, sorted_route, s.top)
+            d = torch.empty(R, W, **f32)
+            m.gemv_act(gu, self.w_down, d, R, W, s.ff, 2 * s.ff, s.ff, sorted_expert, self.w_down.stride(0), 3, p0=s.limit, p1=self.ALPHA)
+        else:
+            xs = torch.empty(R, W, dtype=m.torch_dtype, device=dev)
+            _call("mrs_hyb_moe_gather", h32, sorted_route, None, s.top, xs, R, W, m.dt)
+            gu = m.grouped_linear(xs, self.w_gu, bounds, sorted_expert)
+            act = torch.empty(R, s.ff, dtype=m.torch_dtype, device=dev)
+            _call("mrs_hyb_glu_clamped", gu, act, R, s.ff, s.limit, self.ALPHA, m.dt)
+            d = m.grouped_linear(act, self.w_down, bounds, sorted_expert)
+        sh = None
+        if s.shared_ff:
+            sgu = m.linear(h, self.ws_gu)
+            if T <= m.GEMV_ROWS:
+                sh = torch.empty(T, W, **f32)
+                m.gemv_act(sgu, self.ws_down, sh, T, W, s.shared_ff, 2 * s.shared_ff, s.shared_ff, None, 0, 3, p0=s.shared_limit, p1=self.ALPHA)
+            else:
+                sact = torch.empty(T, s.shared_ff, dtype=m.torch_dtype, device=dev)
+                _call("mrs_hyb_glu_clamped", sgu, sact, T, s.shared_ff, s.shared_limit, self.ALPHA, m.dt)
+                sh = m.linear(sact, self.ws_down)
+        _call("mrs_hyb_moe_combine_weighted", x, d, route_pos, wts, s.top, sh, T, W, int(accumulate))
+
+
+class XieluFeedForward(_Module):
+    """down(act(up h + b_up)) + b_down with act = xIELU: z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1 / 2 + softplus(q)) (e^z - 1 - z) + z / 2; p, q = the tensor `act`."""
+
+    def __init__(self, model, spec: DenseSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+
+    def load(self, get):
+        s, p, W = self.s, self.p, self.m.spec.width
+        self.w_up, self.w_down = self.w(get, p + "up", True), self.w(get, p + "down", True)
+        self.b_up, self.out_bias = self.w(get, p + "up.b", False), self.w(get, p + "down.b", False)
+        if tuple(self.w_up.shape) != (s.ff, W) or tuple(self.w_down.shape) != (W, s.ff):
+            raise ValueError(f"{p}: projection shapes do not match the layer's sizes")
+        pq = np.asarray(get(p + "act").to(torch.float32).cpu().numpy(), dtype=np.float32).reshape(-1)
+        sp = lambda v: np.float32(max(v, np.float32(0))) + np.log1p(np.exp(-np.abs(np.float32(v)), dtype=np.float32), dtype=np.float32)
+        self.ap, self.an = float(sp(pq[0])), float(np.float32(0.5) + sp(pq[1]))
+
+    def forward(self, h, h32, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T = b.rows
+        u = m.linear(h, self.w_up)
+        if T <= m.GEMV_ROWS:   # decode-sized steps: bias and activation in the down product's operand load
+            m.gemv_act(u, self.w_down, x, T, x.shape[1], s.ff, u.stride(0), s.ff, None, 0, 4, bias=self.b_up, p0=self.ap, p1=self.an, accumulate=accumulate)
+            return
+        a = torch.empty(T, s.ff, dtype=m.torch_dtype, device=m.device)
+        _call("mrs_hyb_bias_xielu", u, u.stride(0), self.b_up, a, T, s.ff, self.ap, self.an, m.dt)
+        m.linear(a, self.w_down, out=x, accumulate=accumulate)
+
+
+MIXERS: Dict[str, Callable] = {"mamba2": Mamba2Mixer, "attention": WindowAttention, "talk_attention": TalkSigmoidAttention}
+FEED_FORWARDS: Dict[str, Callable] = {"moe": SigmoidMoe, "moe_softmax_clamped": ClampedSoftmaxMoe, "dense_xielu": XieluFeedForward}
 
 
 class _Layer:
     def __init__(self, model, ls: LayerSpec):
         self.spec = ls
         self.mixer = MIXERS[ls.kind](model, ls.mixer, ls.prefix + "mix.")
-        self.ff = FEED_FORWARDS["moe"](model, ls.ff, ls.prefix + "mlp.") if ls.ff else None
-        self.norm1 = self.norm2 = None
+        self.ff = FEED_FORWARDS[ls.ff.kind](model, ls.ff, ls.prefix + "mlp.") if ls.ff else None
+        self.norm1 = self.norm2 = self.norm1b = self.norm2b = None   # (weight, bias | None)
 
 
 # ------------------------------------------------------------------------------------------------------------------ the model
@@ -432,21 +673,24 @@ class HybridDecoder:
 
     @property
     def has_paged_kv(self) -> bool:
-        return any(isinstance(l.mixer, WindowAttention) for l in self.layers)
+        return any(hasattr(l.mixer, "k_cache") for l in self.layers)
 
     def load_weights(self, get: Callable[[str], torch.Tensor]) -> None:
         sp = self.spec
         f32 = lambda n: get(n).to(self.device, torch.float32).contiguous()
         self.embed = get(sp.embed).to(self.device, self.torch_dtype).contiguous()
         self.head = get(sp.head).to(self.device, self.torch_dtype).contiguous()
-        self.final_norm = f32(sp.final_norm)
+        norm = lambda n: (f32(n), f32(n + ".b") if sp.norm == "layer" else None)
+        self.final_norm = norm(sp.final_norm)
         if tuple(self.embed.shape) != (sp.vocab, sp.width) or tuple(self.head.shape) != (sp.vocab, sp.width):
             raise ValueError("embedding / head shapes do not match vocab x width")
         for l in self.layers:
-            l.norm1 = f32(l.spec.prefix + "norm1")
+            l.norm1 = norm(l.spec.prefix + "norm1")
+            l.norm1b = norm(l.spec.prefix + "norm1b") if sp.post_norms else None
             l.mixer.load(get)
             if l.ff:
-                l.norm2 = f32(l.spec.prefix + "norm2")
+                l.norm2 = norm(l.spec.prefix + "norm2")
+                l.norm2b = norm(l.spec.prefix + "norm2b") if sp.post_norms else None
                 l.ff.load(get)
 
     @classmethod
@@ -468,6 +712,32 @@ class HybridDecoder:
         out32 = torch.empty(rows, width, dtype=torch.float32, device=self.device) if want32 else None
         _call("mrs_hyb_rmsnorm", x, x.stride(0), w, out, out32, None, rows, width, parts, self.spec.eps, int(one_plus), self.dt, gate, gate.stride(0) if gate is not None else 0)
         return (out, out32) if want32 else out
+
+    def layer_norm(self, x, wb, want32: bool = False):
+        """(x - mean) / sqrt(var + eps) * w + b of every row, in the serving dtype (and in f32 with want32)."""
+        rows, width = x.shape
+        out = torch.empty(rows, width, dtype=self.torch_dtype, device=self.device)
+        out32 = torch.empty(rows, width, dtype=torch.float32, device=self.device) if want32 else None
+        _call("mrs_hyb_layernorm", x, x.stride(0), None, wb[0], wb[1], out, out32, None, 0, rows, width, self.spec.eps, self.dt)
+        return (out, out32) if want32 else out
+
+    def pre_norm(self, x, wb, want32: bool = False):
+        """The norm in front of a sublayer (and of the head), of the kind the model's description names."""
+        if self.spec.norm == "layer":
+            return self.layer_norm(x, wb, want32)
+        return self.norm(x, wb[0], one_plus=True, want32=want32)
+
+    def add_post_norm(self, x, y, in_bias, wb) -> None:
+        """x += norm(y + in_bias): a sublayer's product (its bias still to be added) joins the f32 residual stream through the norm behind the sublayer."""
+        if self.spec.norm != "layer":
+            raise NotImplementedError("norms behind a sublayer exist as layer norms only")
+        _call("mrs_hyb_layernorm", y, y.stride(0), in_bias, wb[0], wb[1], None, None, x, x.stride(0), y.shape[0], y.shape[1], self.spec.eps, self.dt)
+
+    def gemv_act(self, a, w, out, M, N, K, lda, ldw, row_group, wstride, in_mode, src_row=None, src_div=1, bias=None, p0=0.0, p1=0.0, accumulate=False, src_scale=None):
+        """out [M, N] (+)= act(a) . w^T for at most GEMV_ROWS rows (or one weight slab per row with `row_group`), the activation evaluated in the operand load.  in_mode:
+        0 plain, 1 silu(gate) * up of a = f32 [gate | up], 2 gathered (and scaled) f32 source rows, 3 clamped GLU of a = f32 [gate | up] (p0 = limit, p1 = the sigmoid's
+        factor), 4 xIELU(a + bias) (p0, p1 = its two coefficients)."""
+        _call("mrs_hyb_gemv_act", a, w, out, M, N, K, lda, ldw, out.stride(0), self.dt, int(accumulate), row_group, wstride, in_mode, src_row, src_scale, src_div, bias, p0, p1)
 
     def linear(self, a, w, out=None, accumulate: bool = False, dtype_code: Optional[int] = None):
         """out (f32 [M, N]) (+)= a [M, K] . w [N, K]^T"""
@@ -510,11 +780,20 @@ class HybridDecoder:
             return torch.empty(0, sp.vocab, dtype=torch.float32, device=self.device)
         x = torch.empty(T, sp.width, dtype=torch.float32, device=self.device)
         _call("mrs_hyb_embed", b.tokens, self.embed, x, T, sp.width, sp.vocab, self.dt)
+        y = torch.empty_like(x) if sp.post_norms else None   # a sublayer's product on its way through the norm behind it
         for l in self.layers:
-            l.mixer.forward(self.norm(x, l.norm1, one_plus=True), x, b)
+            if sp.post_norms:
+                l.mixer.forward(self.pre_norm(x, l.norm1), y, b, accumulate=False)
+                self.add_post_norm(x, y, l.mixer.out_bias, l.norm1b)
+            else:
+                l.mixer.forward(self.pre_norm(x, l.norm1), x, b)
             if l.ff:
-                h, h32 = self.norm(x, l.norm2, one_plus=True, want32=True)
-                l.ff.forward(h, h32, x, b)
+                h, h32 = self.pre_norm(x, l.norm2, want32=True)
+                if sp.post_norms:
+                    l.ff.forward(h, h32, y, b, accumulate=False)
+                    self.add_post_norm(x, y, l.ff.out_bias, l.norm2b)
+                else:
+                    l.ff.forward(h, h32, x, b)
             if self.trace_layers is not None:
                 self.trace_layers.append(x.clone())
         n = b.want.numel()
@@ -522,7 +801,7 @@ class HybridDecoder:
             return torch.empty(0, sp.vocab, dtype=torch.float32, device=self.device)
         xs = torch.empty(n, sp.width, dtype=torch.float32, device=self.device)
         _call("mrs_hyb_gather_rows", x, b.want, xs, n, sp.width)
-        return self.linear(self.norm(xs, self.final_norm, one_plus=True), self.head)
+        return self.linear(self.pre_norm(xs, self.final_norm), self.head)
 
     # ---- decode steps as a HIP graph
     def capture_decode(self, entries: int, max_blocks: int) -> "DecodeGraph":
@@ -531,8 +810,7 @@ class HybridDecoder:
 
     # ---- sizes
     def kv_bytes_per_token(self) -> int:
-        e = 2 if self.dtype == "bfloat16" else 4
-        return sum(e * l.mixer.s.kv_heads * (l.mixer.s.dim + l.mixer.s.vdim) for l in self.layers if isinstance(l.mixer, WindowAttention))
+        return sum(l.mixer.kv_bytes_per_token() for l in self.layers if hasattr(l.mixer, "kv_bytes_per_token"))
 
     def state_bytes_per_slot(self) -> int:
         return sum(l.mixer.state_bytes_per_slot() for l in self.layers if isinstance(l.mixer, Mamba2Mixer))
@@ -554,7 +832,7 @@ class DecodeGraph:
             o += k
         rows = torch.arange(n + 1, dtype=torch.int32, device=dev)   # one row = one segment per entry
         self.batch = RaggedBatch(n, n, mb, v[0], v[1], v[2], v[3], v[4], v[5], v[6].view(n, mb), self._slots, rows[:n].clone(), n, rows[:n], rows[:n],
-                                 torch.ones(n, dtype=torch.int32, device=dev), rows)
+                                 torch.ones(n, dtype=torch.int32, device=dev), rows, 1)
         self._host = np.zeros(self._ints.numel(), dtype=np.int32)
         self._host[3 * n:3 * n + n + 1] = np.arange(n + 1)          # seq_start: one row per entry
         self._host[2 * n:3 * n] = 1                                  # positions >= 1 during warm-up: the slots' states are read, nothing is reset
@@ -563,8 +841,7 @@ class DecodeGraph:
         # warm-up outside capture (lazy module loads).  It really runs -- on state slot 0 and page slot 0, which may belong to a live sequence: put both back afterwards
         keep = []
         for l in model.layers:
-            mx = l.mixer
-            keep += [(t, t[0].clone()) for t in ((mx.conv_state, mx.ssm_state) if isinstance(mx, Mamba2Mixer) else (mx.k_cache, mx.v_cache))]
+            keep += [(t, t[0].clone()) for t in l.mixer.carried()]
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -605,31 +882,52 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
     W = spec.width
     g = torch.Generator(device=device).manual_seed(seed)
     shapes: Dict[str, tuple] = {spec.embed: (spec.vocab, W), spec.head: (spec.vocab, W), spec.final_norm: (W,)}
+    norm_names = {spec.final_norm}
     for ls in spec.layers:
         p, m = ls.prefix, ls.mixer
-        shapes[p + "norm1"] = (W,)
-        if isinstance(m, Mamba2Spec):
+        for n in ["norm1"] + (["norm2"] if ls.ff else []) + ((["norm1b"] + (["norm2b"] if ls.ff else [])) if spec.post_norms else []):
+            norm_names.add(p + n)
+        if isinstance(m, TalkAttentionSpec):
+            shapes.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.q.b": (m.heads * m.dim,), p + "mix.g": (m.heads, W), p + "mix.talk": (m.heads, m.heads),
+                           p + "mix.pb": (m.heads,), p + "mix.o": (W, m.heads * m.vdim), p + "mix.o.b": (W,)})
+            if m.kv_from is None:
+                shapes.update({p + "mix.k": (m.kv_heads * m.dim, W), p + "mix.k.b": (m.kv_heads * m.dim,), p + "mix.v": (m.kv_heads * m.vdim, W), p + "mix.v.b": (m.kv_heads * m.vdim,)})
+        elif isinstance(m, Mamba2Spec):
             shapes.update({p + "mix.in": (2 * m.inner + 2 * m.groups * m.state + m.heads, W), p + "mix.conv": (m.conv_channels, m.conv), p + "mix.conv.b": (m.conv_channels,),
                            p + "mix.dt_bias": (m.heads,), p + "mix.A_log": (m.heads,), p + "mix.D": (m.heads,), p + "mix.norm": (m.inner,), p + "mix.o": (W, m.inner)})
         else:
             shapes.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.kv_heads * m.dim, W), p + "mix.v": (m.kv_heads * m.vdim, W), p + "mix.q.norm": (m.heads * m.dim,),
                            p + "mix.k.norm": (m.kv_heads * m.dim,), p + "mix.o": (W, m.heads * m.vdim)})
-        if ls.ff:
+        if isinstance(ls.ff, DenseSpec):
+            shapes.update({p + "mlp.up": (ls.ff.ff, W), p + "mlp.up.b": (ls.ff.ff,), p + "mlp.down": (W, ls.ff.ff), p + "mlp.down.b": (W,), p + "mlp.act": (2,)})
+        elif ls.ff:
             f = ls.ff
-            shapes[p + "norm2"], shapes[p + "mlp.router"] = (W,), (f.experts, W)
+            shapes[p + "mlp.router"] = (f.experts, W)
             for e in range(f.experts):
                 shapes.update({f"{p}mlp.e{e}.gate": (f.ff, W), f"{p}mlp.e{e}.up": (f.ff, W), f"{p}mlp.e{e}.down": (W, f.ff)})
             if f.shared_ff:
-                shapes.update({p + "mlp.shared.gate": (f.shared_ff, W), p + "mlp.shared.up": (f.shared_ff, W), p + "mlp.shared.down": (W, f.shared_ff), p + "mlp.shared.sg": (1, W)})
+                shapes.update({p + "mlp.shared.gate": (f.shared_ff, W), p + "mlp.shared.up": (f.shared_ff, W), p + "mlp.shared.down": (W, f.shared_ff)})
+                if isinstance(f, MoeSpec):
+                    shapes[p + "mlp.shared.sg"] = (1, W)
+    for n in norm_names:
+        shapes[n] = (W,)
+        if spec.norm == "layer":
+            shapes[n + ".b"] = (W,)
 
     def get(name: str) -> torch.Tensor:
         shape = shapes[name]
         r = torch.randn(*shape, device=device, generator=g)
         last = name.rsplit(".", 1)[-1]
-        if name.endswith(("q.norm", "k.norm")) or last == "D" or name.endswith("mix.norm"):
+        if name.endswith(("q.norm", "k.norm")) or last == "D" or name.endswith("mix.norm") or (name in norm_names and spec.norm == "layer"):
             r = 1.0 + 0.1 * r
-        elif last in ("norm1", "norm2") or name == spec.final_norm:
+        elif name in norm_names:
             r = 0.1 * r
+        elif last == "talk":
+            r = torch.eye(shape[0], device=device) + 0.1 * r
+        elif last == "pb":
+            r = -3.0 + 0.5 * r     # un-normalised weights: most keys weigh little
+        elif last == "act":
+            r = 0.5 * r
         elif last == "dt_bias":
             r = -2.0 + 0.5 * r
         elif last == "A_log":
@@ -644,7 +942,7 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
     return get
 
 
-SPEC_READERS: Dict[str, Callable[[dict], HybridSpec]] = {"Gekilix": gekilix_spec}
+SPEC_READERS: Dict[str, Callable[[dict], HybridSpec]] = {"Gekilix": gekilix_spec, "Sobunex": sobunex_spec}
 
 
 class HybridCache:

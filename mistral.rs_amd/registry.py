@@ -22,6 +22,12 @@ def _load_gekilix(path: str, device, dtype: str = "bfloat16", **kw):
     return HybridDecoder.from_pretrained(path, device, dtype, **kw)
 
 
+@register("Sobunex")
+def _load_sobunex(path: str, device, dtype: str = "bfloat16", **kw):
+    from .hybrid import HybridDecoder
+    return HybridDecoder.from_pretrained(path, device, dtype, **kw)
+
+
 @register("llama")
 def _load_llama_gguf(path: str, device, dtype: str = "bfloat16", **kw):
     from .gguf.archive import load_llama
