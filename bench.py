@@ -706,6 +706,147 @@ def hybrid_leg(a, dev):
                       "config": {"model": out["model"], "global_batch": 1, "seq_len": 512, "parallelism": "tp1"}, "hybrid": out}), flush=True)
 
 
+SOBUNEX_SIZES = {
+    # layer lists that resemble a small and a mid-size decoder: every second layer reads the K / V pages of the layer before it and has routed experts, the others are dense
+    "s": dict(width=1024, layers=8, heads=16, kv=4, dim=64, vdim=64, window=1024, experts=32, top=4, ff=512, shared=1024, dense_ff=4096, vocab=32000),
+    "m": dict(width=2048, layers=8, heads=16, kv=4, dim=128, vdim=128, window=2048, experts=64, top=6, ff=768, shared=2048, dense_ff=8192, vocab=32000),
+    "l": dict(width=4096, layers=4, heads=32, kv=8, dim=128, vdim=128, window=4096, experts=64, top=6, ff=1024, shared=2048, dense_ff=14336, vocab=32000),
+}
+
+
+def sobunex_leg(a, dev):
+    """`--sobunex SIZE`: prefill and decode throughput of a Sobunex layer list (sigmoid attention with mixed head scores, layer norms around every sublayer, xIELU and
+    clamped-GLU softmax-routed feed-forwards; bf16 weights, random) beside the closest model of the package at equal size: a Gekilix list of windowed softmax attention
+    layers with sigmoid-routed experts (same width, depth, heads, head sizes, window, expert count / size, vocabulary).  Then the kernels of the two designs that do like
+    work, one launch each at the model's shapes: time, and the fraction of the roofline (8 TB/s for what a kernel must read and write; the attention kernels run on the
+    vector ALU in both designs, their prompt passes are priced in FLOP/s of the work done)."""
+    import torch
+    from mistralrs_amd.hybrid import (AttentionSpec, ClampedMoeSpec, DenseSpec, HybridCache, HybridDecoder, HybridSpec, LayerSpec, MoeSpec, RaggedBatch, RotarySpec,
+                                      TalkAttentionSpec, _call, synthetic_weights)
+    z = SOBUNEX_SIZES[a.sobunex]
+    W, H, G, D, Dv, win = z["width"], z["heads"], z["kv"], z["dim"], z["vdim"], z["window"]
+    new_layers, old_layers = [], []
+    for i in range(z["layers"]):
+        shared = i % 2 == 1
+        new_layers.append(LayerSpec("talk_attention", TalkAttentionSpec(H, G, D, Dv, D ** -0.5, win, 0.3, 128, i - 1 if shared else None),
+                                    ClampedMoeSpec(z["experts"], z["top"], z["ff"], 7.0, 1.5, z["shared"], 7.0) if shared else DenseSpec(z["dense_ff"]), f"l{i}."))
+        old_layers.append(LayerSpec("attention", AttentionSpec(H, G, D, Dv, D ** -0.5, win, 0, RotarySpec(D // 2, 500000.0, None)),
+                                    MoeSpec(z["experts"], z["top"], z["ff"], z["shared"]), f"l{i}."))
+    specs = {"sobunex": HybridSpec(z["vocab"], W, 1e-6, new_layers, norm="layer", post_norms=True), "gekilix_attention_moe": HybridSpec(z["vocab"], W, 1e-6, old_layers)}
+    prompts, batches, bs, ctx = [512, 2048], [1, 8], 32, 512
+    max_tok = max(prompts) + a.warmup + a.steps + 64
+    blocks_per_seq = -(-(2 * win + 64) // bs)   # the single-kernel runs below place their queries one window deep
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    out = {"sizes": z, "dtype": "bf16", "weights": "random, drawn on the device", "models": {}, "kernels": {}}
+    keep = {}
+    with torch.no_grad():
+        for name, spec in specs.items():
+            model = HybridDecoder(spec, dev, "bfloat16", num_blocks=max(batches) * max(-(-max_tok // bs) + 1, blocks_per_seq) + 2, block_size=bs, state_slots=max(batches))
+            model.load_weights(synthetic_weights(spec, dev, 0))
+            cache = HybridCache(model)
+            r = {"prefill": {}, "decode": {}}
+            for T in prompts:
+                assert cache.reserve(1, T)
+                b = RaggedBatch.build([cache.entry(1, [(1000 + i) % z["vocab"] for i in range(T)], 0, [T - 1])], bs, dev)
+                t = timed(lambda: model.forward_batch(b), 3)
+                r["prefill"][str(T)] = {"tokens_per_sec": round(T / t, 1), "ms": round(1e3 * t, 3)}
+                cache.release(1)
+            for nb in batches:
+                for q in range(nb):
+                    assert cache.reserve(q + 1, ctx + a.warmup + a.steps + 2)
+                model.forward_batch(RaggedBatch.build([cache.entry(q + 1, [(1000 + i + q) % z["vocab"] for i in range(ctx)], 0, []) for q in range(nb)], bs, dev))
+                g = model.capture_decode(nb, -(-(ctx + a.warmup + a.steps + 2) // bs))
+                pos = ctx
+
+                def step():
+                    nonlocal pos
+                    g.replay([cache.entry(q + 1, [7 + q], pos) for q in range(nb)])
+                    pos += 1
+                for _ in range(a.warmup):
+                    step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(a.steps):
+                    step()
+                torch.cuda.synchronize()
+                t = (time.perf_counter() - t0) / a.steps
+                r["decode"][f"batch{nb}"] = {"tokens_per_sec": round(nb / t, 1), "ms_per_step": round(1e3 * t, 4)}
+                del g
+                for q in range(nb):
+                    cache.release(q + 1)
+            out["models"][name] = r
+            keep[name] = model.layers[0].mixer
+            del model, cache
+            torch.cuda.empty_cache()
+        # ---- like kernels of the two designs, one launch each
+        new, old = keep["sobunex"], keep["gekilix_attention_moe"]
+        m = new.m
+        e = 2
+        kern = out["kernels"]
+        for label, nseq, p0, n in (("attention_prompt", 1, 0, 2048), ("attention_prompt_deep", 1, win, 512), ("attention_decode_batch8", 8, win + 17, 1), ("attention_decode_batch1", 1, win + 17, 1)):
+            ents = [{"tokens": [0] * n, "pos0": p0, "slot": 0, "blocks": list(range(1 + q * blocks_per_seq, 1 + (q + 1) * blocks_per_seq)), "want": []} for q in range(nseq)]
+            if ents[-1]["blocks"][-1] >= m.num_blocks:
+                continue
+            b = RaggedBatch.build(ents, bs, dev)
+            T = b.rows
+            qn = torch.randn(T, H * D, device=dev).to(torch.bfloat16)
+            gate = torch.randn(T, H, device=dev)
+            o = torch.empty(T, H * Dv, dtype=torch.bfloat16, device=dev)
+            for c in (new.k_cache, new.v_cache, old.k_cache, old.v_cache):
+                c.normal_()
+            ks = min(new.KEY_SPLITS, -(-min(win, b.max_blocks * bs) // 64)) if T <= new.SPLIT_ROWS else 0   # as the mixer does: few rows share their keys between workgroups
+            scratch = torch.empty(max(ks, 1), T, H * Dv, device=dev)
+            t_new = timed(lambda: _call("mrs_hyb_paged_talk_sigmoid_attn", qn, new.k_cache, new.v_cache, b.block_tables, b.tok_pos, new.talk, new.pb, new.slopes, gate, H, o, T, H, G, D,
+                                        Dv, bs, b.max_blocks, win, D ** -0.5, 1, b.seg_entry, b.seg_row0, b.seg_len, b.segments, b.seg_rows, scratch if ks > 1 else None, ks), 5)
+            t_old = timed(lambda: _call("mrs_hyb_paged_window_attn", qn, old.k_cache, old.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, H, G, D, Dv, bs, b.max_blocks, win, 0,
+                                        D ** -0.5, 1, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT), 5)
+            pairs = sum(min(p0 + i + 1, win) for i in range(n)) * nseq               # visible (query, key) pairs
+            flops = 2.0 * pairs * H * (D + Dv)
+            kv_bytes = nseq * e * G * (D + Dv) * min(p0 + n, win + n - 1) + T * e * H * (D + Dv)
+            kern[label] = {"rows": T, "flops": flops, "min_bytes": kv_bytes,
+                           "sobunex": {"us": round(1e6 * t_new, 1), "tflops": round(flops / t_new / 1e12, 2), "hbm_frac": round(kv_bytes / t_new / HBM_PEAK, 4)},
+                           "gekilix": {"us": round(1e6 * t_old, 1), "tflops": round(flops / t_old / 1e12, 2), "hbm_frac": round(kv_bytes / t_old / HBM_PEAK, 4)},
+                           "time_ratio": round(t_new / t_old, 2)}
+        T = 2048
+        x = torch.randn(T, W, device=dev)
+        wv, bv = torch.randn(W, device=dev), torch.randn(W, device=dev)
+        ob, o32 = torch.empty(T, W, dtype=torch.bfloat16, device=dev), torch.empty(T, W, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_layernorm", x, W, None, wv, bv, ob, o32, None, 0, T, W, 1e-6, 1), 10)
+        t_old = timed(lambda: _call("mrs_hyb_rmsnorm", x, W, wv, ob, o32, None, T, W, 1, 1e-6, 1, 1, None, 0), 10)
+        nb_ = T * W * (4 + 2 + 4)
+        kern["norm_2048_rows"] = {"min_bytes": nb_, "sobunex_layernorm": {"us": round(1e6 * t_new, 1), "hbm_frac": round(nb_ / t_new / HBM_PEAK, 4)},
+                                  "gekilix_rmsnorm": {"us": round(1e6 * t_old, 1), "hbm_frac": round(nb_ / t_old / HBM_PEAK, 4)}, "time_ratio": round(t_new / t_old, 2)}
+        E, top = z["experts"], z["top"]
+        wr = torch.randn(E + 1, W, device=dev)
+        ids, wts, gt = torch.empty(T * top, dtype=torch.int32, device=dev), torch.empty(T * top, device=dev), torch.empty(T, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_route_softmax_topk", x, wr, T, W, E, top, 1.5, ids, wts), 10)
+        t_old = timed(lambda: _call("mrs_hyb_route_sigmoid_topk", x, wr, T, W, E, top, 1, ids, wts, gt), 10)
+        nb_ = T * W * 4 + E * W * 4
+        kern["router_2048_rows"] = {"min_bytes": nb_, "sobunex_softmax": {"us": round(1e6 * t_new, 1), "hbm_frac": round(nb_ / t_new / HBM_PEAK, 4)},
+                                    "gekilix_sigmoid": {"us": round(1e6 * t_old, 1), "hbm_frac": round(nb_ / t_old / HBM_PEAK, 4)}, "time_ratio": round(t_new / t_old, 2)}
+        R, ff = T * top, z["ff"]
+        gu = torch.randn(R, 2 * ff, device=dev)
+        act = torch.empty(R, ff, dtype=torch.bfloat16, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_glu_clamped", gu, act, R, ff, 7.0, 1.702, 1), 10)
+        t_old = timed(lambda: _call("mrs_hyb_glu_silu", gu, act, R, ff, 1), 10)
+        nb_ = R * ff * (8 + 2)
+        kern["glu_prompt"] = {"min_bytes": nb_, "sobunex_clamped": {"us": round(1e6 * t_new, 1), "hbm_frac": round(nb_ / t_new / HBM_PEAK, 4)},
+                              "gekilix_silu": {"us": round(1e6 * t_old, 1), "hbm_frac": round(nb_ / t_old / HBM_PEAK, 4)}, "time_ratio": round(t_new / t_old, 2)}
+    d1 = out["models"]["sobunex"]["decode"]["batch1"]
+    print(json.dumps({"metric": "sobunex_decode_tokens_per_sec", "value": d1["tokens_per_sec"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": d1["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"model": f"sobunex-{a.sobunex}", "global_batch": 1, "seq_len": 512, "parallelism": "tp1"}, "sobunex": out}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -732,7 +873,17 @@ def main():
                     help="instead of the default workload: a layer-list decoder (state-space + windowed-attention mixers, routed experts; bf16) of the given size beside the Llama runner at equal size")
     ap.add_argument("--hybrid-no-llama", action="store_true", help="--hybrid: skip the equal-size Llama leg (profiling runs)")
     ap.add_argument("--hybrid-quick", action="store_true", help="--hybrid: the equal-size Llama leg at the short prompt only")
+    ap.add_argument("--sobunex", choices=sorted(SOBUNEX_SIZES), default=None,
+                    help="instead of the default workload: a Sobunex layer list (sigmoid attention with mixed head scores, dense / routed feed-forwards; bf16) of the given size beside "
+                         "a windowed-attention + routed-experts list of the package at equal size, and the like kernels of the two one by one")
     a = ap.parse_args()
+    if a.sobunex:
+        import torch
+        dev = torch.device("cuda", 0)
+        torch.cuda.set_device(dev)
+        if a.steps == 256:
+            a.steps = 128
+        return sobunex_leg(a, dev)
     if a.hybrid:
         import torch
         dev = torch.device("cuda", 0)

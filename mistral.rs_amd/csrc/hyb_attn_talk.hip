@@ -8,7 +8,10 @@
 // head.  Keys go by in passes of 64:
 //   A  wave w scores heads w, w + 4, ..: a lane = a key, its row is read in 16-byte loads and multiplied with the NQ query vectors in LDS      -> s [H][64][NQ] (LDS)
 //   B  a thread = (4 output heads, key, query): sum over g with talk^T rows as float4 broadcasts, visibility, sigmoid                            -> p [H][64][NQ] (LDS)
-//   C  a thread = IT x (head, value pair): the value pair of key j is read once and added into the NQ accumulators (registers)
+//   C  a thread = IT x (head, VW values): the values of key j are read once (one 16-byte load when VW = 8) and added into the NQ accumulators (registers).  When there
+//      are fewer (head, value group) items than threads, JS thread groups share the keys of a pass (j = group, group + JS, ..) and their sums meet in LDS at the end
+// Few rows (decoded tokens): the passes are dealt to KS workgroups per tile (grid.z); since the sum over keys has no normaliser the partial sums simply add -- they go to
+// an f32 scratch [KS][rows][H * Dv] and a second kernel adds them in a fixed order, applies the gate and rounds.
 // Grouped heads: query head h reads key / value head h / (H / G).
 #include "common.cuh"
 #include <float.h>
@@ -32,6 +35,8 @@ struct TalkArgs {
   const int *seg_entry, *seg_row0, *seg_len;
   int ldg, H, G, D, Dv, block_size, max_blocks, window, vec_k, vec_v;
   float scale;
+  float *scratch;           // key splits > 1: [splits][rows][H * Dv] partial sums (no gate)
+  int rows, pass_per_split;
 };
 
 template <class T> struct TLd;
@@ -55,7 +60,7 @@ template <> struct TLd<float> {
   static __device__ __forceinline__ void v2(const float *p, float &x, float &y) { const float2 v = *(const float2 *)p; x = v.x; y = v.y; }
 };
 
-template <class T, int NQ, int IT> __global__ void __launch_bounds__(256) talk_sigmoid_attn_kernel(TalkArgs a) {
+template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256) talk_sigmoid_attn_kernel(TalkArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int z = blockIdx.y;
@@ -83,19 +88,32 @@ template <class T, int NQ, int IT> __global__ void __launch_bounds__(256) talk_s
   int lo = a.window > 0 ? i0 - a.window + 1 : 0;
   if (lo < 0) lo = 0;
   const int hi = i0 + nq - 1, total = hi - lo + 1;
-  const int Dvh = (Dv + 1) >> 1, items = H * Dvh;
-  float o[IT][NQ][2];
+  const int DvG = (Dv + VW - 1) / VW, items = H * DvG;   // (head, group of VW values)
+  int JS = 1;                                            // thread groups that share a pass's keys
+  while (JS < 8 && items * JS * 2 <= 256 * IT) JS <<= 1;
+  int it_h[IT], it_d[IT], it_j[IT];                      // a thread's items: head, first value, key group (-1: none)
+  float o[IT][NQ][VW];
 #pragma unroll
-  for (int u = 0; u < IT; ++u)
+  for (int u = 0; u < IT; ++u) {
+    const int sidx = tid + u * 256, item = sidx % items, jp = sidx / items;
+    it_h[u] = item / DvG;
+    it_d[u] = (item - it_h[u] * DvG) * VW;
+    it_j[u] = jp < JS ? jp : -1;
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) o[u][q][0] = o[u][q][1] = 0.f;
+    for (int q = 0; q < NQ; ++q)
+#pragma unroll
+      for (int e = 0; e < VW; ++e) o[u][q][e] = 0.f;
+  }
+  const int v_lo = blockIdx.z * a.pass_per_split * 64;
+  int v_hi = v_lo + a.pass_per_split * 64;
+  if (v_hi > total) v_hi = total;
 
-  for (int v0 = 0; v0 < total; v0 += 64) {
+  for (int v0 = v_lo; v0 < v_hi; v0 += 64) {
     if (tid < 64) {
       const int key = lo + v0 + tid;
       base0[tid] = key <= hi ? (long long)bt[key / bs] * a.G * bs + key % bs : -1;
     }
-    __syncthreads();  // also: q and talk are in LDS (first pass); the previous pass has consumed p and the row indices
+    __syncthreads();  // also: q and talk are in LDS (first pass)
     // ---- A: raw scores with the distance bias
     {
       const long long b0 = base0[lane];
@@ -155,70 +173,105 @@ template <class T, int NQ, int IT> __global__ void __launch_bounds__(256) talk_s
     }
     __syncthreads();
     // ---- C: weighted value sums
-    const int cnt = total - v0 < 64 ? total - v0 : 64;
+    const int cnt = v_hi - v0 < 64 ? v_hi - v0 : 64;
 #pragma unroll
     for (int u = 0; u < IT; ++u) {
-      const int item = tid + u * 256;
-      if (item < items) {
-        const int h = item / Dvh, d = (item - h * Dvh) << 1;
-        const T *vb = (const T *)a.v_cache + (size_t)(h / rep) * bs * Dv + d;
-        const float *ph = pw + (size_t)h * 64 * NQ;
-        const bool two = d + 1 < Dv;
-#pragma unroll 2
-        for (int j = 0; j < cnt; ++j) {
-          const T *vr = vb + (size_t)base0[j] * Dv;
-          float x, y = 0.f;
-          if (a.vec_v) TLd<T>::v2(vr, x, y);
-          else { x = to_f<T>(vr[0]); if (two) y = to_f<T>(vr[1]); }
-          float pj[NQ];
-          if (NQ >= 4) {
+      if (it_j[u] < 0) continue;
+      const int h = it_h[u], d = it_d[u];
+      const T *vb = (const T *)a.v_cache + (size_t)(h / rep) * bs * Dv + d;
+      const float *ph = pw + (size_t)h * 64 * NQ;
+#pragma unroll 4
+      for (int j = it_j[u]; j < cnt; j += JS) {
+        const T *vr = vb + (size_t)base0[j] * Dv;
+        float x[VW];
+        if (VW == 8) TLd<T>::v8(vr, x);
+        else if (a.vec_v) TLd<T>::v2(vr, x[0], x[1]);
+        else { x[0] = to_f<T>(vr[0]); x[1] = d + 1 < Dv ? to_f<T>(vr[1]) : 0.f; }
+        float pj[NQ];
+        if (NQ >= 4) {
 #pragma unroll
-            for (int q4 = 0; q4 < NQ; q4 += 4) {
-              const float4 p4 = *(const float4 *)(ph + j * NQ + q4);
-              pj[q4] = p4.x; pj[q4 + 1] = p4.y; pj[q4 + 2] = p4.z; pj[q4 + 3] = p4.w;
-            }
-          } else {
-#pragma unroll
-            for (int q = 0; q < NQ; ++q) pj[q] = ph[j * NQ + q];
+          for (int q4 = 0; q4 < NQ; q4 += 4) {
+            const float4 p4 = *(const float4 *)(ph + j * NQ + q4);
+            pj[q4] = p4.x; pj[q4 + 1] = p4.y; pj[q4 + 2] = p4.z; pj[q4 + 3] = p4.w;
           }
+        } else {
 #pragma unroll
-          for (int q = 0; q < NQ; ++q) {
-            o[u][q][0] = fmaf(pj[q], x, o[u][q][0]);
-            o[u][q][1] = fmaf(pj[q], y, o[u][q][1]);
-          }
+          for (int q = 0; q < NQ; ++q) pj[q] = ph[j * NQ + q];
         }
+#pragma unroll
+        for (int q = 0; q < NQ; ++q)
+#pragma unroll
+          for (int e = 0; e < VW; ++e) o[u][q][e] = fmaf(pj[q], x[e], o[u][q][e]);
       }
     }
     __syncthreads();  // p and the row indices of this pass are consumed
   }
+  if (JS > 1) {  // the key groups' sums meet in LDS (everything else there has been consumed), one query at a time; group 0 keeps the total
+    float *red = lds;  // [256 * IT][VW]
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < IT; ++u)
+        if (it_j[u] > 0)
+#pragma unroll
+          for (int e = 0; e < VW; ++e) red[(size_t)(tid + u * 256) * VW + e] = o[u][q][e];
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < IT; ++u)
+        if (it_j[u] == 0)
+          for (int p = 1; p < JS; ++p)
+#pragma unroll
+            for (int e = 0; e < VW; ++e) o[u][q][e] += red[(size_t)(tid + u * 256 + p * items) * VW + e];
+    }
+  }
 #pragma unroll
   for (int u = 0; u < IT; ++u) {
-    const int item = tid + u * 256;
-    if (item >= items) continue;
-    const int h = item / Dvh, d = (item - h * Dvh) << 1;
+    if (it_j[u] != 0) continue;
+    const int h = it_h[u], d = it_d[u];
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
       if (q >= nq) break;
-      const float gl = a.gate ? 1.0f / (1.0f + expf(-a.gate[(size_t)(t0 + q) * a.ldg + h])) : 1.0f;
-      T *out = (T *)a.out + ((size_t)(t0 + q) * H + h) * Dv + d;
-      out[0] = from_f<T>(o[u][q][0] * gl);
-      if (d + 1 < Dv) out[1] = from_f<T>(o[u][q][1] * gl);
+      if (a.scratch) {
+        float *out = a.scratch + ((size_t)blockIdx.z * a.rows + (t0 + q)) * H * Dv + (size_t)h * Dv + d;
+#pragma unroll
+        for (int e = 0; e < VW; ++e)
+          if (d + e < Dv) out[e] = o[u][q][e];
+      } else {
+        const float gl = a.gate ? 1.0f / (1.0f + expf(-a.gate[(size_t)(t0 + q) * a.ldg + h])) : 1.0f;
+        T *out = (T *)a.out + ((size_t)(t0 + q) * H + h) * Dv + d;
+#pragma unroll
+        for (int e = 0; e < VW; ++e)
+          if (d + e < Dv) out[e] = from_f<T>(o[u][q][e] * gl);
+      }
     }
   }
 }
 
-template <class T, int NQ, int IT> static int launch_talk(const TalkArgs &a, dim3 grid, size_t lds, hipStream_t st) {
+// the key splits' partial sums, added in split order; gate; rounding
+template <class T> __global__ void __launch_bounds__(256) talk_reduce_kernel(const float *__restrict__ scratch, int splits, int rows, int HDv, int Dv, const float *__restrict__ gate,
+                                                                             int ldg, T *__restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, n = (size_t)rows * HDv;
+  if (i >= n) return;
+  const int t = (int)(i / HDv), c = (int)(i - (size_t)t * HDv);
+  float acc = 0.f;
+  for (int k = 0; k < splits; ++k) acc += scratch[(size_t)k * n + i];
+  const float gl = gate ? 1.0f / (1.0f + expf(-gate[(size_t)t * ldg + c / Dv])) : 1.0f;
+  out[i] = from_f<T>(acc * gl);
+}
+
+template <class T, int NQ, int IT, int VW> static int launch_talk(const TalkArgs &a, dim3 grid, size_t lds, hipStream_t st) {
   if (lds > 65536) {
     static thread_local size_t granted = 0;  // per instantiation
     if (lds > granted) {
-      if (hipFuncSetAttribute((const void *)talk_sigmoid_attn_kernel<T, NQ, IT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      if (hipFuncSetAttribute((const void *)talk_sigmoid_attn_kernel<T, NQ, IT, VW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return tfail("mrs_hyb_paged_talk_sigmoid_attn: the heads' queries and scores do not fit into LDS");
       }
       granted = lds;
     }
   }
-  hipLaunchKernelGGL((talk_sigmoid_attn_kernel<T, NQ, IT>), grid, dim3(256), lds, st, a);
+  hipLaunchKernelGGL((talk_sigmoid_attn_kernel<T, NQ, IT, VW>), grid, dim3(256), lds, st, a);
   return 0;
 }
 
@@ -229,44 +282,75 @@ using namespace mrs::hyb;
 
 extern "C" const char *mrs_hyb_talk_last_error() { return g_terr; }
 
-/* Rows are addressed through the batch's segment table (seg_entry / seg_row0 / seg_len [segments], at most seg_rows rows each: 1 when every entry brings one decoded token).  gate [rows, ldg]: logits whose sigmoid
- * multiplies the head outputs (nullable).  talk [H, H], pb [H], slopes [H] f32 on the device. */
+/* Rows are addressed through the batch's segment table (seg_entry / seg_row0 / seg_len [segments], at most seg_rows rows each: 1 when every entry brings one decoded token).
+ * gate [rows, ldg]: logits whose sigmoid multiplies the head outputs (nullable).  talk [H, H], pb [H], slopes [H] f32 on the device.  scratch (nullable): f32
+ * [scratch_splits][rows][H * Dv]; with it, a step of few workgroups deals every tile's keys to up to scratch_splits workgroups. */
 extern "C" int mrs_hyb_paged_talk_sigmoid_attn(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_pos, const float *talk,
                                                const float *pb, const float *slopes, const float *gate, int ldg, void *out, int rows, int H, int G, int D, int Dv, int block_size,
                                                int max_blocks, int window, float scale, int dtype, const int *seg_entry, const int *seg_row0, const int *seg_len, int segments,
-                                               int seg_rows, void *stream) {
+                                               int seg_rows, float *scratch, int scratch_splits, void *stream) {
   if (rows <= 0 || segments <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0) return tfail("mrs_hyb_paged_talk_sigmoid_attn: head sizes (heads % kv_heads == 0)");
   if (!seg_entry || !seg_row0 || !seg_len || seg_rows <= 0 || segments > 65535) return tfail("mrs_hyb_paged_talk_sigmoid_attn: the segment table is missing or too long");
   if (dtype != 1 && dtype != 2) return tfail("mrs_hyb_paged_talk_sigmoid_attn: dtype");
   const int esz = dtype == 1 ? 2 : 4;
+  const int vw = (Dv % 8 == 0 && ((uintptr_t)v_cache % 16) == 0) ? 8 : 2;
   TalkArgs a{q, k_cache, v_cache, block_tables, tok_pos, talk, pb, slopes, gate, out, seg_entry, seg_row0, seg_len, ldg, H, G, D, Dv, block_size, max_blocks, window,
-             (D % 8 == 0 && ((uintptr_t)k_cache % 16) == 0) ? 1 : 0, (Dv % 2 == 0 && ((uintptr_t)v_cache % (2 * esz)) == 0) ? 1 : 0, scale};
-  const int items = H * ((Dv + 1) / 2);
+             (D % 8 == 0 && ((uintptr_t)k_cache % 16) == 0) ? 1 : 0, (Dv % 2 == 0 && ((uintptr_t)v_cache % (2 * esz)) == 0) ? 1 : 0, scale, nullptr, rows, 1 << 24};
+  const int items = H * ((Dv + vw - 1) / vw);
   int it = (items + 255) / 256;
   it = it <= 1 ? 1 : (it <= 2 ? 2 : (it <= 4 ? 4 : 8));
-  if (items > 8 * 256) return tfail("mrs_hyb_paged_talk_sigmoid_attn: heads * value size above 4096");
-  const int Dp = (D + 7) & ~7, Hp = (H + 3) & ~3;
-  auto lds_of = [&](int nq) { return ((size_t)H * nq * Dp + 2 * (size_t)H * 64 * nq + (size_t)H * Hp) * 4 + 64 * 8; };
+  if (items > 8 * 256) return tfail("mrs_hyb_paged_talk_sigmoid_attn: heads * value size too large for one workgroup");
+  const int Dp = (D + 7) & ~7, Hp = (H + 3) & ~3, cap = vw == 8 ? 8 : 16;   // accumulator registers: NQ * IT * VW <= 64 (32 for pairs)
+  auto lds_of = [&](int nq) {
+    const size_t work = ((size_t)H * nq * Dp + 2 * (size_t)H * 64 * nq + (size_t)H * Hp) * 4 + 64 * 8, red = (size_t)256 * it * vw * 4;
+    return work > red ? work : red;
+  };
   int nq = 1;
-  if (seg_rows > 1)  // some entry brings a portion: the widest tile that keeps the accumulators in registers and the scores in 64 KB of LDS
+  if (seg_rows > 1)  // some entry brings a portion: the widest tile that keeps the accumulators in registers and leaves room for two workgroups' LDS per compute unit
     for (int c = 8; c > 1; c >>= 1)
-      if (c * it <= 16 && c <= seg_rows && lds_of(c) <= 65536) { nq = c; break; }
+      if (c * it <= cap && c <= seg_rows && lds_of(c) <= 72 * 1024) { nq = c; break; }
+  if (nq * it > cap) return tfail("mrs_hyb_paged_talk_sigmoid_attn: heads * value size too large for one workgroup");
+  if (vw == 2 && nq == 8) nq = 4;   // pairs: tiles of 1, 2 and 4 queries
   const size_t lds = lds_of(nq);
   if (lds > 160 * 1024) return tfail("mrs_hyb_paged_talk_sigmoid_attn: the heads' queries and scores do not fit into LDS");
-  dim3 grid((seg_rows + nq - 1) / nq, segments);
+  const int tiles = (seg_rows + nq - 1) / nq;
+  int splits = 1;
+  if (scratch && scratch_splits > 1 && (long long)tiles * segments < 256) {
+    const long long ctx = (long long)max_blocks * block_size, span = window > 0 && window + nq - 1 < ctx ? window + nq - 1 : ctx;
+    const int passes = (int)((span + 63) / 64), want = (int)((512 + (long long)tiles * segments - 1) / ((long long)tiles * segments));
+    splits = passes < want ? passes : want;
+    if (splits > scratch_splits) splits = scratch_splits;
+    if (splits > 1) {
+      a.pass_per_split = (passes + splits - 1) / splits;
+      splits = (passes + a.pass_per_split - 1) / a.pass_per_split;
+    }
+    if (splits > 1) a.scratch = scratch;
+  }
+  dim3 grid(tiles, segments, splits);
   hipStream_t st = (hipStream_t)stream;
   int rc = 1;
-#define MRS_TALK_IT(T, NQ_) (it == 1 ? launch_talk<T, NQ_, 1>(a, grid, lds, st) : it == 2 ? launch_talk<T, NQ_, 2>(a, grid, lds, st) : tfail("mrs_hyb_paged_talk_sigmoid_attn: tile"))
+#define MRS_TALK_L(T, NQ_, IT_, VW_) rc = launch_talk<T, NQ_, IT_, VW_>(a, grid, lds, st)
 #define MRS_TALK(T) do { \
-    if (nq == 8) rc = MRS_TALK_IT(T, 8); \
-    else if (nq == 4) rc = it <= 2 ? MRS_TALK_IT(T, 4) : launch_talk<T, 4, 4>(a, grid, lds, st); \
-    else if (nq == 2) rc = it <= 2 ? MRS_TALK_IT(T, 2) : (it == 4 ? launch_talk<T, 2, 4>(a, grid, lds, st) : launch_talk<T, 2, 8>(a, grid, lds, st)); \
-    else rc = it <= 2 ? MRS_TALK_IT(T, 1) : (it == 4 ? launch_talk<T, 1, 4>(a, grid, lds, st) : launch_talk<T, 1, 8>(a, grid, lds, st)); } while (0)
+    if (vw == 8) { \
+      if (nq == 8) MRS_TALK_L(T, 8, 1, 8); \
+      else if (nq == 4) { if (it == 1) MRS_TALK_L(T, 4, 1, 8); else MRS_TALK_L(T, 4, 2, 8); } \
+      else if (nq == 2) { if (it == 1) MRS_TALK_L(T, 2, 1, 8); else if (it == 2) MRS_TALK_L(T, 2, 2, 8); else MRS_TALK_L(T, 2, 4, 8); } \
+      else { if (it == 1) MRS_TALK_L(T, 1, 1, 8); else if (it == 2) MRS_TALK_L(T, 1, 2, 8); else if (it == 4) MRS_TALK_L(T, 1, 4, 8); else MRS_TALK_L(T, 1, 8, 8); } \
+    } else { \
+      if (nq == 4) { if (it == 1) MRS_TALK_L(T, 4, 1, 2); else if (it == 2) MRS_TALK_L(T, 4, 2, 2); else MRS_TALK_L(T, 4, 4, 2); } \
+      else if (nq == 2) { if (it == 1) MRS_TALK_L(T, 2, 1, 2); else if (it == 2) MRS_TALK_L(T, 2, 2, 2); else if (it == 4) MRS_TALK_L(T, 2, 4, 2); else MRS_TALK_L(T, 2, 8, 2); } \
+      else { if (it == 1) MRS_TALK_L(T, 1, 1, 2); else if (it == 2) MRS_TALK_L(T, 1, 2, 2); else if (it == 4) MRS_TALK_L(T, 1, 4, 2); else MRS_TALK_L(T, 1, 8, 2); } \
+    } } while (0)
   if (dtype == 1) MRS_TALK(mrs::bf16_t); else MRS_TALK(float);
 #undef MRS_TALK
-#undef MRS_TALK_IT
+#undef MRS_TALK_L
   if (rc) return rc;
+  if (splits > 1) {
+    const size_t n = (size_t)rows * H * Dv;
+    if (dtype == 1) hipLaunchKernelGGL(talk_reduce_kernel<mrs::bf16_t>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, scratch, splits, rows, H * Dv, Dv, gate, ldg, (mrs::bf16_t *)out);
+    else hipLaunchKernelGGL(talk_reduce_kernel<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, scratch, splits, rows, H * Dv, Dv, gate, ldg, (float *)out);
+  }
   if (hipGetLastError() != hipSuccess) return tfail("mrs_hyb_paged_talk_sigmoid_attn: launch failed");
   return 0;
 }

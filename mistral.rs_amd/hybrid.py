@@ -49,7 +49,7 @@ _SIGS = {
     "mrs_hyb_bias_xielu": [_vp, _i, _vp, _vp, _i, _i, _f, _f, _i, _vp],
     "mrs_hyb_layernorm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp],
     "mrs_hyb_qkv_bias_temp_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp],
-    "mrs_hyb_paged_talk_sigmoid_attn": [_vp] * 9 + [_i, _vp] + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _vp],
+    "mrs_hyb_paged_talk_sigmoid_attn": [_vp] * 9 + [_i, _vp] + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _vp, _i, _vp],
     "mrs_hyb_gemm": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _l, _i, _vp],
     "mrs_hyb_gemv": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp],
     "mrs_hyb_gemv_act": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp, _f, _f, _vp],
@@ -434,6 +434,8 @@ class TalkSigmoidAttention(_Module):
     (q *= 1 + coef ln(floor((pos + 1) / every) + 1)) and a per-head distance bias.  Head g scores key j as scale (q_g . k_j) - 2^(-8 (g + 1) / heads) (i - j); the heads'
     scores are mixed by the [heads, heads] matrix `talk`; a key with 0 <= i - j < window weighs sigmoid(mixed + pb_h), un-normalised; head outputs are multiplied by
     sigmoid(gate logit), then projected.  With `kv_from` the layer has no key / value projections: it reads the K / V pages of that earlier layer (same block tables)."""
+    KEY_SPLITS = 64      # at most this many workgroups share a row's keys
+    SPLIT_ROWS = 128     # steps of at most this many rows may split
 
     def __init__(self, model, spec: TalkAttentionSpec, prefix: str):
         super().__init__(model)
@@ -479,8 +481,12 @@ class TalkSigmoidAttention(_Module):
               s.dim, s.vdim, m.block_size, s.temp_coef, s.temp_every, m.dt)
         src = self if s.kv_from is None else m.layers[s.kv_from].mixer      # that layer ran earlier in this step: its pages hold this step's rows already
         o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
+        # a step of few rows deals every row's keys to several workgroups: room for their partial sums
+        splits = min(self.KEY_SPLITS, -(-(min(s.window, b.max_blocks * m.block_size) if s.window > 0 else b.max_blocks * m.block_size) // 64)) if T <= self.SPLIT_ROWS else 0
+        scratch = torch.empty(splits, T, s.heads * s.vdim, dtype=torch.float32, device=m.device) if splits > 1 else None
         _call("mrs_hyb_paged_talk_sigmoid_attn", q, src.k_cache, src.v_cache, b.block_tables, b.tok_pos, self.talk, self.pb, self.slopes, u[:, self.gate_col:], u.stride(0), o,
-              T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, b.max_blocks, s.window, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, b.seg_rows)
+              T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, b.max_blocks, s.window, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, b.seg_rows,
+              scratch, splits)
         m.linear(o, self.w_o, out=x, accumulate=accumulate)
 
 
