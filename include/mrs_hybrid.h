@@ -32,6 +32,7 @@ int mrs_hyb_moe_combine_weighted(float *out, const float *d, const int *route_po
 int mrs_hyb_glu_clamped(const float *gu, void *out, int rows, int ff, float limit, float alpha, int dtype, void *stream);
 int mrs_hyb_bias_xielu(const float *u, int ldu, const float *bias, void *out, int rows, int ff, float ap, float an, int dtype, void *stream);
 int mrs_hyb_layernorm(const float *x, int ldx, const float *in_bias, const float *w, const float *b, void *out, float *out32, float *resid, int ldr, int rows, int width, float eps, int dtype, void *stream);
+int mrs_hyb_layernorm_pair(const float *y, int ldy, const float *in_bias, const float *w, const float *b, float *resid, int ldr, const float *w2, const float *b2, void *out, float *out32, int rows, int width, float eps, int dtype, void *stream);
 int mrs_hyb_qkv_bias_temp_cache(const float *qkv, int ld, const float *qb, const float *kb, const float *vb, const int *tok_pos, const long long *slot_mapping, void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int block_size, float temp_coef, int temp_every, int dtype, void *stream);
 /* ---- hyb_attn_talk.hip */
 const char *mrs_hyb_talk_last_error();

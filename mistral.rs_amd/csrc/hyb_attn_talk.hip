@@ -15,6 +15,7 @@
 // Grouped heads: query head h reads key / value head h / (H / G).
 #include "common.cuh"
 #include <float.h>
+#include <stdlib.h>
 
 namespace mrs {
 namespace hyb {
@@ -60,7 +61,7 @@ template <> struct TLd<float> {
   static __device__ __forceinline__ void v2(const float *p, float &x, float &y) { const float2 v = *(const float2 *)p; x = v.x; y = v.y; }
 };
 
-template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256) talk_sigmoid_attn_kernel(TalkArgs a) {
+template <class T, int NQ, int IT, int VW, int NT> __global__ void __launch_bounds__(NT) talk_sigmoid_attn_kernel(TalkArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int z = blockIdx.y;
@@ -76,11 +77,11 @@ template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256
   float *tk = pw + (size_t)H * 64 * NQ;     // [H][Hp]: tk[g][h] = talk[h][g]
   long long *base0 = (long long *)(tk + (size_t)H * Hp);  // [64]: page row of the pass's keys for key / value head 0 (-1: past the end)
   const int s = a.seg_entry[z], i0 = a.tok_pos[t0];
-  for (int e = tid; e < H * NQ * Dp; e += 256) {
+  for (int e = tid; e < H * NQ * Dp; e += NT) {
     const int g = e / (NQ * Dp), r = e - g * NQ * Dp, q = r / Dp, d = r - q * Dp;
     qs[e] = (q < nq && d < D) ? to_f<T>(((const T *)a.q)[((size_t)(t0 + q) * H + g) * D + d]) : 0.f;
   }
-  for (int e = tid; e < H * Hp; e += 256) {
+  for (int e = tid; e < H * Hp; e += NT) {
     const int g = e / Hp, h = e - g * Hp;
     tk[e] = h < H ? a.talk[(size_t)h * H + g] : 0.f;
   }
@@ -90,12 +91,12 @@ template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256
   const int hi = i0 + nq - 1, total = hi - lo + 1;
   const int DvG = (Dv + VW - 1) / VW, items = H * DvG;   // (head, group of VW values)
   int JS = 1;                                            // thread groups that share a pass's keys
-  while (JS < 8 && items * JS * 2 <= 256 * IT) JS <<= 1;
+  while (JS < 8 && items * JS * 2 <= NT * IT) JS <<= 1;
   int it_h[IT], it_d[IT], it_j[IT];                      // a thread's items: head, first value, key group (-1: none)
   float o[IT][NQ][VW];
 #pragma unroll
   for (int u = 0; u < IT; ++u) {
-    const int sidx = tid + u * 256, item = sidx % items, jp = sidx / items;
+    const int sidx = tid + u * NT, item = sidx % items, jp = sidx / items;
     it_h[u] = item / DvG;
     it_d[u] = (item - it_h[u] * DvG) * VW;
     it_j[u] = jp < JS ? jp : -1;
@@ -118,7 +119,7 @@ template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256
     {
       const long long b0 = base0[lane];
       const int key = lo + v0 + lane;
-      for (int g = wave; g < H; g += 4) {
+      for (int g = wave; g < H; g += NT / 64) {
         float acc[NQ];
 #pragma unroll
         for (int q = 0; q < NQ; ++q) acc[q] = 0.f;
@@ -155,7 +156,7 @@ template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256
     }
     __syncthreads();
     // ---- B: mix the heads, visibility, sigmoid
-    for (int it = tid; it < (Hp >> 2) * 64 * NQ; it += 256) {
+    for (int it = tid; it < (Hp >> 2) * 64 * NQ; it += NT) {
       const int jq = it % (64 * NQ), h0 = (it / (64 * NQ)) << 2;
       const int j = jq / NQ, q = jq - j * NQ;
       float m0 = 0.f, m1 = 0.f, m2 = 0.f, m3 = 0.f;
@@ -207,7 +208,7 @@ template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256
     __syncthreads();  // p and the row indices of this pass are consumed
   }
   if (JS > 1) {  // the key groups' sums meet in LDS (everything else there has been consumed), one query at a time; group 0 keeps the total
-    float *red = lds;  // [256 * IT][VW]
+    float *red = lds;  // [NT * IT][VW]
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
       __syncthreads();
@@ -215,14 +216,14 @@ template <class T, int NQ, int IT, int VW> __global__ void __launch_bounds__(256
       for (int u = 0; u < IT; ++u)
         if (it_j[u] > 0)
 #pragma unroll
-          for (int e = 0; e < VW; ++e) red[(size_t)(tid + u * 256) * VW + e] = o[u][q][e];
+          for (int e = 0; e < VW; ++e) red[(size_t)(tid + u * NT) * VW + e] = o[u][q][e];
       __syncthreads();
 #pragma unroll
       for (int u = 0; u < IT; ++u)
         if (it_j[u] == 0)
           for (int p = 1; p < JS; ++p)
 #pragma unroll
-            for (int e = 0; e < VW; ++e) o[u][q][e] += red[(size_t)(tid + u * 256 + p * items) * VW + e];
+            for (int e = 0; e < VW; ++e) o[u][q][e] += red[(size_t)(tid + u * NT + p * items) * VW + e];
     }
   }
 #pragma unroll
@@ -260,18 +261,18 @@ template <class T> __global__ void __launch_bounds__(256) talk_reduce_kernel(con
   out[i] = from_f<T>(acc * gl);
 }
 
-template <class T, int NQ, int IT, int VW> static int launch_talk(const TalkArgs &a, dim3 grid, size_t lds, hipStream_t st) {
+template <class T, int NQ, int IT, int VW, int NT> static int launch_talk(const TalkArgs &a, dim3 grid, size_t lds, hipStream_t st) {
   if (lds > 65536) {
     static thread_local size_t granted = 0;  // per instantiation
     if (lds > granted) {
-      if (hipFuncSetAttribute((const void *)talk_sigmoid_attn_kernel<T, NQ, IT, VW>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      if (hipFuncSetAttribute((const void *)talk_sigmoid_attn_kernel<T, NQ, IT, VW, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
         (void)hipGetLastError();
         return tfail("mrs_hyb_paged_talk_sigmoid_attn: the heads' queries and scores do not fit into LDS");
       }
       granted = lds;
     }
   }
-  hipLaunchKernelGGL((talk_sigmoid_attn_kernel<T, NQ, IT, VW>), grid, dim3(256), lds, st, a);
+  hipLaunchKernelGGL((talk_sigmoid_attn_kernel<T, NQ, IT, VW, NT>), grid, dim3(NT), lds, st, a);
   return 0;
 }
 
@@ -298,18 +299,20 @@ extern "C" int mrs_hyb_paged_talk_sigmoid_attn(const void *q, const void *k_cach
   TalkArgs a{q, k_cache, v_cache, block_tables, tok_pos, talk, pb, slopes, gate, out, seg_entry, seg_row0, seg_len, ldg, H, G, D, Dv, block_size, max_blocks, window,
              (D % 8 == 0 && ((uintptr_t)k_cache % 16) == 0) ? 1 : 0, (Dv % 2 == 0 && ((uintptr_t)v_cache % (2 * esz)) == 0) ? 1 : 0, scale, nullptr, rows, 1 << 24};
   const int items = H * ((Dv + vw - 1) / vw);
-  int it = (items + 255) / 256;
+  const int nt = (vw == 8 && H >= 8) ? 512 : 256;   // eight waves when there are heads for them: twice the waves per byte of LDS
+  int it = (items + nt - 1) / nt;
   it = it <= 1 ? 1 : (it <= 2 ? 2 : (it <= 4 ? 4 : 8));
-  if (items > 8 * 256) return tfail("mrs_hyb_paged_talk_sigmoid_attn: heads * value size too large for one workgroup");
+  if (items > 8 * nt) return tfail("mrs_hyb_paged_talk_sigmoid_attn: heads * value size too large for one workgroup");
+  static const int lds_kb = getenv("MRS_TALK_LDS_KB") ? atoi(getenv("MRS_TALK_LDS_KB")) : 79;   // tile choice: LDS per workgroup (79: two workgroups per compute unit)
   const int Dp = (D + 7) & ~7, Hp = (H + 3) & ~3, cap = vw == 8 ? 8 : 16;   // accumulator registers: NQ * IT * VW <= 64 (32 for pairs)
   auto lds_of = [&](int nq) {
-    const size_t work = ((size_t)H * nq * Dp + 2 * (size_t)H * 64 * nq + (size_t)H * Hp) * 4 + 64 * 8, red = (size_t)256 * it * vw * 4;
+    const size_t work = ((size_t)H * nq * Dp + 2 * (size_t)H * 64 * nq + (size_t)H * Hp) * 4 + 64 * 8, red = (size_t)nt * it * vw * 4;
     return work > red ? work : red;
   };
   int nq = 1;
   if (seg_rows > 1)  // some entry brings a portion: the widest tile that keeps the accumulators in registers and leaves room for two workgroups' LDS per compute unit
     for (int c = 8; c > 1; c >>= 1)
-      if (c * it <= cap && c <= seg_rows && lds_of(c) <= 72 * 1024) { nq = c; break; }
+      if (c * it <= cap && c <= seg_rows && lds_of(c) <= (size_t)lds_kb * 1024) { nq = c; break; }
   if (nq * it > cap) return tfail("mrs_hyb_paged_talk_sigmoid_attn: heads * value size too large for one workgroup");
   if (vw == 2 && nq == 8) nq = 4;   // pairs: tiles of 1, 2 and 4 queries
   const size_t lds = lds_of(nq);
@@ -330,7 +333,7 @@ extern "C" int mrs_hyb_paged_talk_sigmoid_attn(const void *q, const void *k_cach
   dim3 grid(tiles, segments, splits);
   hipStream_t st = (hipStream_t)stream;
   int rc = 1;
-#define MRS_TALK_L(T, NQ_, IT_, VW_) rc = launch_talk<T, NQ_, IT_, VW_>(a, grid, lds, st)
+#define MRS_TALK_L(T, NQ_, IT_, VW_) do { if (VW_ == 8 && nt == 512) rc = launch_talk<T, NQ_, IT_, VW_, (VW_ == 8 ? 512 : 256)>(a, grid, lds, st); else rc = launch_talk<T, NQ_, IT_, VW_, 256>(a, grid, lds, st); } while (0)
 #define MRS_TALK(T) do { \
     if (vw == 8) { \
       if (nq == 8) MRS_TALK_L(T, 8, 1, 8); \

@@ -821,9 +821,11 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(float *__restrict__ x,
 
 // ---------------------------------------------------------------------------------- layer norm with weight and bias: (v - mean) / sqrt(mean((v - mean)^2) + eps) * w + b
 // v = x (+ in_bias): the bias of the product that made x.  The result goes to out (T) and / or out32, and / or is ADDED to resid (the f32 residual stream: norms after a sublayer).
+// With w2: the updated residual row is normed once more (weights w2, b2: the norm in front of the NEXT sublayer) and THAT goes to out / out32 -- two launches and a pass
+// over the stream less per sublayer.
 template <class T> __global__ void __launch_bounds__(256) layernorm_kernel(const float *__restrict__ x, int ldx, const float *__restrict__ in_bias, const float *__restrict__ w,
                                                                            const float *__restrict__ b, T *__restrict__ out, float *__restrict__ out32, float *__restrict__ resid, int ldr,
-                                                                           int width, float eps) {
+                                                                           int width, float eps, const float *__restrict__ w2, const float *__restrict__ b2) {
   __shared__ float red[4];
   extern __shared__ float row[];
   const int t = blockIdx.x;
@@ -841,6 +843,28 @@ template <class T> __global__ void __launch_bounds__(256) layernorm_kernel(const
     q = fmaf(dv, dv, q);
   }
   const float inv = 1.0f / sqrtf(block_sum_256(q, red) / (float)width + eps);
+  if (w2) {
+    float s2 = 0.f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+      const float r = resid[(size_t)t * ldr + c] + ((row[c] - mean) * inv * w[c] + (b ? b[c] : 0.f));
+      resid[(size_t)t * ldr + c] = r;
+      row[c] = r;
+      s2 += r;
+    }
+    const float mean2 = block_sum_256(s2, red) / (float)width;
+    float q2 = 0.f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+      const float dv = row[c] - mean2;
+      q2 = fmaf(dv, dv, q2);
+    }
+    const float inv2 = 1.0f / sqrtf(block_sum_256(q2, red) / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += 256) {
+      const float y = (row[c] - mean2) * inv2 * w2[c] + (b2 ? b2[c] : 0.f);
+      if (out) out[(size_t)t * width + c] = from_f<T>(y);
+      if (out32) out32[(size_t)t * width + c] = y;
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < width; c += 256) {
     const float y = (row[c] - mean) * inv * w[c] + (b ? b[c] : 0.f);
     if (out) out[(size_t)t * width + c] = from_f<T>(y);
@@ -1104,10 +1128,25 @@ extern "C" int mrs_hyb_layernorm(const float *x, int ldx, const float *in_bias, 
   if (rows <= 0) return 0;
   if (width <= 0 || width > 15000) return fail("mrs_hyb_layernorm: 1 .. 15000 values per row");
   const size_t lds = (size_t)width * 4;
-  if (dtype == 1) hipLaunchKernelGGL(layernorm_kernel<mrs::bf16_t>, dim3(rows), dim3(256), lds, S_(stream), x, ldx, in_bias, w, b, (mrs::bf16_t *)out, out32, resid, ldr, width, eps);
-  else if (dtype == 2) hipLaunchKernelGGL(layernorm_kernel<float>, dim3(rows), dim3(256), lds, S_(stream), x, ldx, in_bias, w, b, (float *)out, out32, resid, ldr, width, eps);
+  if (dtype == 1) hipLaunchKernelGGL(layernorm_kernel<mrs::bf16_t>, dim3(rows), dim3(256), lds, S_(stream), x, ldx, in_bias, w, b, (mrs::bf16_t *)out, out32, resid, ldr, width, eps,
+                                     (const float *)nullptr, (const float *)nullptr);
+  else if (dtype == 2) hipLaunchKernelGGL(layernorm_kernel<float>, dim3(rows), dim3(256), lds, S_(stream), x, ldx, in_bias, w, b, (float *)out, out32, resid, ldr, width, eps,
+                                          (const float *)nullptr, (const float *)nullptr);
   else return fail("mrs_hyb_layernorm: dtype");
   return ok_or("mrs_hyb_layernorm");
+}
+
+/* resid += norm(y + in_bias; w, b), then out (dtype) / out32 = norm(resid; w2, b2): the norm behind a sublayer and the norm in front of the next one in one pass */
+extern "C" int mrs_hyb_layernorm_pair(const float *y, int ldy, const float *in_bias, const float *w, const float *b, float *resid, int ldr, const float *w2, const float *b2,
+                                      void *out, float *out32, int rows, int width, float eps, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  if (width <= 0 || width > 15000) return fail("mrs_hyb_layernorm_pair: 1 .. 15000 values per row");
+  if (!resid || !w2 || !w) return fail("mrs_hyb_layernorm_pair: the residual stream and both norms' weights are needed");
+  const size_t lds = (size_t)width * 4;
+  if (dtype == 1) hipLaunchKernelGGL(layernorm_kernel<mrs::bf16_t>, dim3(rows), dim3(256), lds, S_(stream), y, ldy, in_bias, w, b, (mrs::bf16_t *)out, out32, resid, ldr, width, eps, w2, b2);
+  else if (dtype == 2) hipLaunchKernelGGL(layernorm_kernel<float>, dim3(rows), dim3(256), lds, S_(stream), y, ldy, in_bias, w, b, (float *)out, out32, resid, ldr, width, eps, w2, b2);
+  else return fail("mrs_hyb_layernorm_pair: dtype");
+  return ok_or("mrs_hyb_layernorm_pair");
 }
 
 /* temp_every <= 0: no query temperature.  k_cache null: the rows carry no key / value columns (a layer that reads another layer's pages) */

@@ -48,6 +48,7 @@ _SIGS = {
     "mrs_hyb_glu_clamped": [_vp, _vp, _i, _i, _f, _f, _i, _vp],
     "mrs_hyb_bias_xielu": [_vp, _i, _vp, _vp, _i, _i, _f, _f, _i, _vp],
     "mrs_hyb_layernorm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp],
+    "mrs_hyb_layernorm_pair": [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     "mrs_hyb_qkv_bias_temp_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp],
     "mrs_hyb_paged_talk_sigmoid_attn": [_vp] * 9 + [_i, _vp] + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _vp, _i, _vp],
     "mrs_hyb_gemm": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _l, _i, _vp],
@@ -733,11 +734,19 @@ class HybridDecoder:
             return self.layer_norm(x, wb, want32)
         return self.norm(x, wb[0], one_plus=True, want32=want32)
 
-    def add_post_norm(self, x, y, in_bias, wb) -> None:
-        """x += norm(y + in_bias): a sublayer's product (its bias still to be added) joins the f32 residual stream through the norm behind the sublayer."""
+    def add_post_norm(self, x, y, in_bias, wb, then=None, want32: bool = False):
+        """x += norm(y + in_bias): a sublayer's product (its bias still to be added) joins the f32 residual stream through the norm behind the sublayer.  `then` = the
+        (weight, bias) of the norm in front of the next sublayer: the same launch norms the updated rows with it and returns them like `pre_norm`."""
         if self.spec.norm != "layer":
             raise NotImplementedError("norms behind a sublayer exist as layer norms only")
-        _call("mrs_hyb_layernorm", y, y.stride(0), in_bias, wb[0], wb[1], None, None, x, x.stride(0), y.shape[0], y.shape[1], self.spec.eps, self.dt)
+        rows, width = y.shape
+        if then is None:
+            _call("mrs_hyb_layernorm", y, y.stride(0), in_bias, wb[0], wb[1], None, None, x, x.stride(0), rows, width, self.spec.eps, self.dt)
+            return None
+        out = torch.empty(rows, width, dtype=self.torch_dtype, device=self.device)
+        out32 = torch.empty(rows, width, dtype=torch.float32, device=self.device) if want32 else None
+        _call("mrs_hyb_layernorm_pair", y, y.stride(0), in_bias, wb[0], wb[1], x, x.stride(0), then[0], then[1], out, out32, rows, width, self.spec.eps, self.dt)
+        return (out, out32) if want32 else out
 
     def gemv_act(self, a, w, out, M, N, K, lda, ldw, row_group, wstride, in_mode, src_row=None, src_div=1, bias=None, p0=0.0, p1=0.0, accumulate=False, src_scale=None):
         """out [M, N] (+)= act(a) . w^T for at most GEMV_ROWS rows (or one weight slab per row with `row_group`), the activation evaluated in the operand load.  in_mode:
@@ -787,18 +796,21 @@ class HybridDecoder:
         x = torch.empty(T, sp.width, dtype=torch.float32, device=self.device)
         _call("mrs_hyb_embed", b.tokens, self.embed, x, T, sp.width, sp.vocab, self.dt)
         y = torch.empty_like(x) if sp.post_norms else None   # a sublayer's product on its way through the norm behind it
-        for l in self.layers:
+        h_next = None                                         # post-norm designs: the next sublayer's input, normed by the launch that closed the previous sublayer
+        for li, l in enumerate(self.layers):
             if sp.post_norms:
-                l.mixer.forward(self.pre_norm(x, l.norm1), y, b, accumulate=False)
-                self.add_post_norm(x, y, l.mixer.out_bias, l.norm1b)
+                l.mixer.forward(h_next if h_next is not None else self.pre_norm(x, l.norm1), y, b, accumulate=False)
+                nxt = self.layers[li + 1].norm1 if li + 1 < len(self.layers) else None
+                if l.ff:
+                    h, h32 = self.add_post_norm(x, y, l.mixer.out_bias, l.norm1b, then=l.norm2, want32=True)
+                    l.ff.forward(h, h32, y, b, accumulate=False)
+                    h_next = self.add_post_norm(x, y, l.ff.out_bias, l.norm2b, then=nxt)
+                else:
+                    h_next = self.add_post_norm(x, y, l.mixer.out_bias, l.norm1b, then=nxt)
             else:
                 l.mixer.forward(self.pre_norm(x, l.norm1), x, b)
-            if l.ff:
-                h, h32 = self.pre_norm(x, l.norm2, want32=True)
-                if sp.post_norms:
-                    l.ff.forward(h, h32, y, b, accumulate=False)
-                    self.add_post_norm(x, y, l.ff.out_bias, l.norm2b)
-                else:
+                if l.ff:
+                    h, h32 = self.pre_norm(x, l.norm2, want32=True)
                     l.ff.forward(h, h32, x, b)
             if self.trace_layers is not None:
                 self.trace_layers.append(x.clone())

@@ -211,7 +211,13 @@ def test_layer_norm_kernel(dev, width):
     assert rel(out32.double().cpu(), want) < 2e-6 and rel(out.double().cpu(), want) < 2e-6
     r = res.to(dev)
     _call("mrs_hyb_layernorm", x.to(dev), width, ib.to(dev), w.to(dev), b.to(dev), None, None, r, width, 9, width, 1e-5, 2)
-    assert rel(r.double().cpu(), res.double() + O.layer_norm((x + ib).double(), w.double(), b.double(), 1e-5)) < 2e-6
+    new = res.double() + O.layer_norm((x + ib).double(), w.double(), b.double(), 1e-5)
+    assert rel(r.double().cpu(), new) < 2e-6
+    # the norm behind a sublayer and the norm in front of the next one in one launch
+    w2, b2 = torch.randn(width, generator=g), torch.randn(width, generator=g)
+    r = res.to(dev)
+    _call("mrs_hyb_layernorm_pair", x.to(dev), width, ib.to(dev), w.to(dev), b.to(dev), r, width, w2.to(dev), b2.to(dev), out, out32, 9, width, 1e-5, 2)
+    assert rel(r.double().cpu(), new) < 2e-6 and rel(out32.double().cpu(), O.layer_norm(new, w2.double(), b2.double(), 1e-5)) < 3e-6 and rel(out.double().cpu(), out32.double().cpu()) == 0
 
 
 @pytest.mark.gpu
