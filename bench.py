@@ -728,8 +728,8 @@ def sobunex_leg(a, dev):
     new_layers, old_layers = [], []
     for i in range(z["layers"]):
         shared = i % 2 == 1
-        new_layers.append(LayerSpec("talk_attention", TalkAttentionSpec(H, G, D, Dv, D ** -0.5, win, 0.3, 128, i - 1 if shared else None),
-                                    ClampedMoeSpec(z["experts"], z["top"], z["ff"], 7.0, 1.5, z["shared"], 7.0) if shared else DenseSpec(z["dense_ff"]), f"l{i}."))
+        new_layers.append(LayerSpec("talk_attention", TalkAttentionSpec(H, G, D, Dv, D ** -0.5, win, 0.25, 256, i - 1 if shared else None),
+                                    ClampedMoeSpec(z["experts"], z["top"], z["ff"], 7.0, 2.0, z["shared"], 7.0) if shared else DenseSpec(z["dense_ff"]), f"l{i}."))
         old_layers.append(LayerSpec("attention", AttentionSpec(H, G, D, Dv, D ** -0.5, win, 0, RotarySpec(D // 2, 500000.0, None)),
                                     MoeSpec(z["experts"], z["top"], z["ff"], z["shared"]), f"l{i}."))
     specs = {"sobunex": HybridSpec(z["vocab"], W, 1e-6, new_layers, norm="layer", post_norms=True), "gekilix_attention_moe": HybridSpec(z["vocab"], W, 1e-6, old_layers)}
@@ -828,7 +828,7 @@ def sobunex_leg(a, dev):
         E, top = z["experts"], z["top"]
         wr = torch.randn(E + 1, W, device=dev)
         ids, wts, gt = torch.empty(T * top, dtype=torch.int32, device=dev), torch.empty(T * top, device=dev), torch.empty(T, device=dev)
-        t_new = timed(lambda: _call("mrs_hyb_route_softmax_topk", x, wr, T, W, E, top, 1.5, ids, wts), 10)
+        t_new = timed(lambda: _call("mrs_hyb_route_softmax_topk", x, wr, T, W, E, top, 2.0, ids, wts), 10)
         t_old = timed(lambda: _call("mrs_hyb_route_sigmoid_topk", x, wr, T, W, E, top, 1, ids, wts, gt), 10)
         nb_ = T * W * 4 + E * W * 4
         kern["router_2048_rows"] = {"min_bytes": nb_, "sobunex_softmax": {"us": round(1e6 * t_new, 1), "hbm_frac": round(nb_ / t_new / HBM_PEAK, 4)},

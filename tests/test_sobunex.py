@@ -25,7 +25,7 @@ def dense(ff=56):
     return {"kind": "dense", "ff": ff}
 
 
-def moe(experts=5, top=2, ff=24, shared=16, scale=1.5, limit=1.0, shared_limit=0.75):
+def moe(experts=5, top=2, ff=24, shared=16, scale=1.25, limit=1.5, shared_limit=0.75):
     return {"kind": "moe", "router": {"experts": experts, "top": top, "scale": scale}, "expert": {"ff": ff, "limit": limit},
             "shared": {"ff": shared, "limit": shared_limit} if shared else None}
 
@@ -334,7 +334,7 @@ def test_planted_keys_at_every_edge(dev, dtype):
     slopes = torch.zeros(H)
     zeros_gate = torch.zeros(64, H, device=dev)               # sigmoid(0) = 1 / 2 on every head output
     blk, off = torch.tensor([blocks[t // bs] for t in range(T)], device=dev), torch.arange(T, device=dev) % bs
-    for size in (40, 290):
+    for size in (37, 290):
         cases = []
         for i in (60, 64, 95, 96, 299):
             for j in (i - size, i - size + 1, 0, i, 31, 32, i - 1, i - 64, i - 65):
@@ -448,7 +448,7 @@ def test_mixed_batches_with_reused_pages_and_slots(dev, dtype, bar):
 
 @pytest.mark.gpu
 def test_long_decoding_past_windows_and_temperature_steps(dev):
-    cfg = config([layer(size=9, every=11), layer(kv_from=0, size=40, every=64, mlp="moe")])
+    cfg = config([layer(size=9, every=11), layer(kv_from=0, size=45, every=64, mlp="moe")])
     w = weights(cfg, 8)
     t = toks(260, cfg["vocab"], 16)
     want = O.forward(cfg, f64(w), t)
@@ -470,6 +470,20 @@ def test_sizes_that_coincide_or_equal_one(dev):
         assert rel(sv.step([(1, t[:1])])[0], want[:1]) < 3e-5
         got = sv.step([(2, t[:1])]) + sv.step([(2, t[1:3])]) + sv.step([(2, t[3:])])
         assert rel(torch.cat(got), want) < 3e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,bar", [("float32", 3e-5), ("bfloat16", 5e-2)])
+def test_sizes_off_every_vector_width(dev, dtype, bar):
+    """width, vocabulary, head sizes, feed-forward and expert sizes that no 16-byte load divides: the element-wise paths of every kernel, prompt and decode"""
+    cfg = config([layer(heads=3, kv_heads=1, dim=11, vdim=13, size=19, every=7, mlp=dense(27)), layer(heads=3, kv_heads=1, dim=11, vdim=13, size=70, kv_from=0, mlp=moe(6, 3, 15, 21)),
+                  layer(heads=5, kv_heads=5, dim=6, vdim=9, size=0, mlp=moe(3, 2, 7, 0))], vocab=77, width=50)
+    w = weights(cfg, 13)
+    t = toks(100, cfg["vocab"], 18)
+    want = O.forward(cfg, f64(w), t)
+    sv = Served(cfg, w, dev, dtype)
+    got = sv.step([(1, t[:67])]) + sv.step([(1, t[67:90])]) + [sv.step([(1, [x])])[0] for x in t[90:]]
+    assert close(torch.cat(got), want, bar)
 
 
 @pytest.mark.gpu
