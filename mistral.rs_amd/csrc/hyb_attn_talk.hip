@@ -4,9 +4,9 @@
 // key (0 <= i - j < window; window <= 0: every j <= i) weighs   p_h = sigmoid(s'_h + pb_h)   -- no normalisation over the keys, so there is no running maximum or sum and
 // the keys can be consumed in any order --   o_h = sum_j p_h v_j,   and the head's output is multiplied by sigmoid(gate logit of (row, h)).  Scores, weights and sums are f32.
 //
-// Because every output head needs the scores of ALL heads, one workgroup owns NQ consecutive rows of one entry (a tile of a segment; NQ = 1 for decoded tokens) for every
-// head.  Keys go by in passes of 64:
-//   A  wave w scores heads w, w + 4, ..: a lane = a key, its row is read in 16-byte loads and multiplied with the NQ query vectors in LDS      -> s [H][64][NQ] (LDS)
+// Because every output head needs the scores of ALL heads, one workgroup (NT = 256 or 512 threads) owns NQ consecutive rows of one entry (a tile of a segment; NQ = 1 for
+// decoded tokens) for every head.  Keys go by in passes of 64:
+//   A  wave w scores heads w, w + NT / 64, ..: a lane = a key, its row is read in 16-byte loads and multiplied with the NQ query vectors in LDS      -> s [H][64][NQ] (LDS)
 //   B  a thread = (4 output heads, key, query): sum over g with talk^T rows as float4 broadcasts, visibility, sigmoid                            -> p [H][64][NQ] (LDS)
 //   C  a thread = IT x (head, VW values): the values of key j are read once (one 16-byte load when VW = 8) and added into the NQ accumulators (registers).  When there
 //      are fewer (head, value group) items than threads, JS thread groups share the keys of a pass (j = group, group + JS, ..) and their sums meet in LDS at the end
