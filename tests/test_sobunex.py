@@ -17,8 +17,6 @@ import mistralrs_amd  # noqa: F401
 from mistralrs_amd import _lib
 from tests import sobunex_oracle as O
 
-HYB = os.path.exists(_lib.path("hybrid"))
-
 
 # ---------------------------------------------------------------------------------------------------------------- configurations and weights
 def dense(ff=56):
